@@ -1,0 +1,69 @@
+"""ctypes binding of ``libfsta.so`` (declarations mirror ``include/fsta.h``)."""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_uint32, c_void_p
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libfsta.so")
+
+F32, F16, BF16 = 0, 1, 2
+OK, EINVAL, EUNSUPPORTED, EHIP = 0, -1, -2, -3
+FLAG_FAST_PV, FLAG_GENERIC = 1, 2
+PRE_TOO_MANY_ANCESTORS, PRE_BAD_NODE_ID, PRE_BAD_LEVEL = 1, 2, 4
+ABI_VERSION = 1
+
+# name -> (restype, argtypes); every symbol include/fsta.h declares
+SIGNATURES = {
+    "fsta_abi_version": (c_int, []),
+    "fsta_last_error": (c_char_p, []),
+    "fsta_mask_words": (c_int32, [c_int32]),
+    "fsta_precompute": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int32, c_int32,
+                                c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "fsta_pack_mask": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p, c_void_p,
+                               c_void_p]),
+    "fsta_attention_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                   c_void_p, c_void_p, c_void_p, c_void_p,
+                                   c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
+                                   c_int32, c_int32, c_int32, c_float, c_uint32, c_void_p]),
+    "fsta_lineage_from_parents": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
+                                          c_void_p]),
+}
+
+_lib = None
+
+
+class FstaError(RuntimeError):
+    """A libfsta entry point returned an error code."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"libfsta error {code}: {message}")
+        self.code = code
+
+
+def load():
+    """Loads the library once; raises if it has not been built.
+
+    There is no CPU fallback: without the HIP library the package cannot compute.
+    """
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m fstattention_amd.build` "
+            "(needs hipcc; the package has no CPU fallback)")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    if lib.fsta_abi_version() != ABI_VERSION:
+        raise ImportError(f"{LIB_PATH}: ABI version {lib.fsta_abi_version()}, expected {ABI_VERSION}")
+    _lib = lib
+    return lib
+
+
+def check(code: int):
+    if code != OK:
+        raise FstaError(code, load().fsta_last_error().decode("utf-8", "replace"))

@@ -1,0 +1,164 @@
+"""``fst_attention``: the operator of reference ``fstattention.py:153-181`` on MI355X.
+
+Same positional signature, same tensor layouts, same two assertions.  The body
+hands raw device pointers to ``libfsta.so`` (hand-written HIP for gfx950) on the
+current torch stream; torch only owns the memory.
+"""
+from __future__ import annotations
+
+from typing import NamedTuple, Optional
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}
+
+
+class PackedTreeMask(NamedTuple):
+    """Bit-packed form of ``ancestor_mask`` the kernels read.
+
+    ``mask_bits`` uint32-as-int32 ``[NB, ceil(A/32), M]`` (bit ``b`` of word ``w``
+    of row ``r`` = ``ancestor_mask[j, r, 32*w + b]``), ``anc_count`` int32 ``[NB]``.
+    """
+    mask_bits: torch.Tensor
+    anc_count: torch.Tensor
+    block_m: int
+    max_ancestors: int
+
+
+def _stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def pack_tree_mask(ancestor_idx: torch.Tensor, ancestor_mask: torch.Tensor) -> PackedTreeMask:
+    """bool ``[NB, M, A]`` mask (+ ``ancestor_idx`` for the ``-1`` slots) -> packed bits."""
+    if not ancestor_mask.is_cuda or not ancestor_idx.is_cuda:
+        raise ValueError("pack_tree_mask needs tensors on the GPU")
+    if ancestor_mask.dtype != torch.bool or ancestor_idx.dtype != torch.int64:
+        raise ValueError("ancestor_mask must be bool and ancestor_idx int64")
+    if ancestor_mask.dim() != 3 or ancestor_idx.dim() != 2 or \
+            ancestor_idx.shape != (ancestor_mask.shape[0], ancestor_mask.shape[2]):
+        raise ValueError(f"shape mismatch: ancestor_idx {tuple(ancestor_idx.shape)}, "
+                         f"ancestor_mask {tuple(ancestor_mask.shape)}")
+    lib = _lib.load()
+    nb, m, a = ancestor_mask.shape
+    ancestor_mask = ancestor_mask.contiguous()
+    ancestor_idx = ancestor_idx.contiguous()
+    dev = ancestor_mask.device
+    words = (a + 31) // 32
+    bits = torch.empty((nb, words, m), dtype=torch.int32, device=dev)
+    count = torch.empty((nb,), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(lib.fsta_pack_mask(ancestor_idx.data_ptr(), ancestor_mask.data_ptr(), nb, m, a,
+                                      bits.data_ptr(), count.data_ptr(), _stream_ptr(dev)))
+    return PackedTreeMask(bits, count, m, a)
+
+
+def _packed_for(ancestor_idx: torch.Tensor, ancestor_mask) -> PackedTreeMask:
+    """Packed mask of a bool tensor, remembered on the tensor object.
+
+    The kernel inputs are built once per decoding step and reused by every
+    layer; the packed copy is kept as an attribute of ``ancestor_mask`` and
+    dropped when either tensor has been written to since (torch's version
+    counters) or ``ancestor_idx`` is a different tensor.
+    """
+    if isinstance(ancestor_mask, PackedTreeMask):
+        return ancestor_mask
+    key = (ancestor_mask._version, ancestor_idx.data_ptr(), ancestor_idx._version,
+           tuple(ancestor_mask.shape))
+    cached = getattr(ancestor_mask, "_fsta_packed", None)
+    if cached is not None and cached[0] == key:
+        return cached[1]
+    packed = pack_tree_mask(ancestor_idx, ancestor_mask)
+    try:
+        ancestor_mask._fsta_packed = (key, packed)
+    except AttributeError:
+        pass
+    return packed
+
+
+def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
+                  BLOCK_M=128, MAX_ANCESTORS=64, *, out_dtype: Optional[torch.dtype] = None,
+                  return_lse: bool = False, fast_pv: bool = False, generic: bool = False):
+    """Fused sparse tree attention forward (reference ``fstattention.py:153-181``).
+
+    ``q [Z,H,Nq,D]``, ``k,v [Z,H,Nk,D]`` (``Nk - Nq`` leading rows are a dense
+    prefix every query sees), ``ancestor_idx`` int64 ``[NB, MAX_ANCESTORS]``,
+    ``ancestor_mask`` bool ``[NB, BLOCK_M, MAX_ANCESTORS]`` (or a
+    :class:`PackedTreeMask`), ``leaf_idx`` int64 ``[NB, BLOCK_M]``; returns
+    ``o`` shaped and typed like ``q``.
+
+    Beyond the reference: ``out_dtype=torch.float32`` keeps the output
+    unrounded, ``return_lse`` also returns the base-2 log-sum-exp ``[Z*H, Nq]``
+    the reference computes and drops (``fstattention.py:139-141,181``),
+    ``fast_pv`` trades accuracy of the bf16 weights for matrix-core time, and
+    ``generic`` forces the scalar kernel.  Inputs the reference silently
+    mis-handles raise ``ValueError`` here (non-contiguous tensors, index
+    tensors whose shapes do not match ``BLOCK_M`` / ``MAX_ANCESTORS``).
+    """
+    # shape constraints (the reference's two assertions)
+    Lq, Lk, Lv = q.shape[-1], k.shape[-1], v.shape[-1]
+    assert Lq == Lk and Lk == Lv
+    assert Lk in {16, 32, 64, 128}
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("q, k, v must be [batch, heads, seq, head_dim]")
+    if not (q.is_cuda and k.is_cuda and v.is_cuda):
+        raise ValueError("fst_attention runs on the GPU only (no CPU fallback); move q/k/v to 'cuda'")
+    if not (q.device == k.device == v.device == ancestor_idx.device == leaf_idx.device):
+        raise ValueError("all tensors must live on the same device")
+    if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ValueError(f"q/k/v must share one dtype of float32/float16/bfloat16, got "
+                         f"{q.dtype}, {k.dtype}, {v.dtype}")
+    if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
+        raise ValueError("q, k, v must be contiguous")
+    Z, H, Nq, D = q.shape
+    if k.shape[:2] != (Z, H) or v.shape != k.shape:
+        raise ValueError(f"k/v shapes {tuple(k.shape)}/{tuple(v.shape)} do not match q {tuple(q.shape)}")
+    Nk = k.shape[2]
+    if Nk < Nq:
+        raise ValueError(f"k has {Nk} rows, fewer than q's {Nq}")
+    nb = -(-Nq // BLOCK_M)
+    if ancestor_idx.dtype != torch.int64 or leaf_idx.dtype != torch.int64:
+        raise ValueError("ancestor_idx and leaf_idx must be int64")
+    if tuple(ancestor_idx.shape) != (nb, MAX_ANCESTORS):
+        raise ValueError(f"ancestor_idx is {tuple(ancestor_idx.shape)}, expected "
+                         f"(ceil(Nq/BLOCK_M)={nb}, MAX_ANCESTORS={MAX_ANCESTORS})")
+    if tuple(leaf_idx.shape) != (nb, BLOCK_M):
+        raise ValueError(f"leaf_idx is {tuple(leaf_idx.shape)}, expected ({nb}, BLOCK_M={BLOCK_M})")
+    if isinstance(ancestor_mask, PackedTreeMask):
+        if (ancestor_mask.block_m, ancestor_mask.max_ancestors) != (BLOCK_M, MAX_ANCESTORS) or \
+                ancestor_mask.mask_bits.shape[0] != nb:
+            raise ValueError("packed mask was built for another block size / ancestor count")
+    elif tuple(ancestor_mask.shape) != (nb, BLOCK_M, MAX_ANCESTORS):
+        raise ValueError(f"ancestor_mask is {tuple(ancestor_mask.shape)}, expected "
+                         f"({nb}, {BLOCK_M}, {MAX_ANCESTORS})")
+    out_dtype = out_dtype or q.dtype
+    if out_dtype not in (q.dtype, torch.float32):
+        raise ValueError("out_dtype must be the input dtype or torch.float32")
+
+    lib = _lib.load()
+    ancestor_idx = ancestor_idx.contiguous()
+    leaf_idx = leaf_idx.contiguous()
+    packed = _packed_for(ancestor_idx, ancestor_mask)
+    o = torch.empty(q.shape, dtype=out_dtype, device=q.device)
+    lse = torch.empty((Z * H, Nq), device=q.device, dtype=torch.float32)
+    flags = (_lib.FLAG_FAST_PV if fast_pv else 0) | (_lib.FLAG_GENERIC if generic else 0)
+    with torch.cuda.device(q.device):
+        _lib.check(lib.fsta_attention_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
+            ancestor_idx.data_ptr(), packed.mask_bits.data_ptr(), packed.anc_count.data_ptr(),
+            leaf_idx.data_ptr(), Z, H, Nq, Nk, D, _DTYPES[q.dtype], _DTYPES[out_dtype],
+            BLOCK_M, MAX_ANCESTORS, nb, float(sm_scale), flags, _stream_ptr(q.device)))
+    return (o, lse) if return_lse else o
+
+
+def shift_for_prefix(ancestor_idx: torch.Tensor, leaf_idx: torch.Tensor, prefix: int):
+    """Index tensors for K/V laid out as ``[prefix | tree]``.
+
+    The reference's caller adds the prefix length to every entry
+    (``fstattention.py:211-212``), which turns the ``-1`` sentinels into the
+    valid row ``prefix-1``; this shifts real entries only.
+    """
+    return (torch.where(ancestor_idx >= 0, ancestor_idx + prefix, ancestor_idx),
+            torch.where(leaf_idx >= 0, leaf_idx + prefix, leaf_idx))

@@ -1,0 +1,78 @@
+"""Builds ``libfsta.so`` (HIP kernels + C ABI) for gfx950 with hipcc.
+
+    python -m fstattention_amd.build
+
+The library is written next to this file so that it travels with the source
+tree; nothing is installed.  hipcc cross-compiles, so no GPU is needed.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(PKG_DIR, "csrc")
+LIB_PATH = os.path.join(PKG_DIR, "libfsta.so")
+OBJ_DIR = os.path.join(PKG_DIR, "csrc", "_obj")
+
+SOURCES = [
+    "fsta_capi.hip",
+    "fsta_precompute.hip",
+    "fsta_attention_generic.hip",
+    "fsta_attention_mfma.hip",
+]
+
+# packed-fp32 VALU forms are switched off for device code on purpose
+HIPCC_FLAGS = [
+    "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option", "-Wno-option-ignored",
+]
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found (set HIPCC or install ROCm)")
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s\n%s" % (" ".join(cmd), proc.stdout, proc.stderr))
+    return proc.stderr
+
+
+def build_library(verbose: bool = True, jobs: int | None = None) -> str:
+    """Compiles every source and links ``libfsta.so``; always rebuilds."""
+    hipcc = _hipcc()
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    jobs = jobs or min(len(SOURCES), os.cpu_count() or 1, 16)
+
+    def compile_one(src):
+        obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
+        warn = _run([hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj])
+        return obj, warn
+
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        results = list(pool.map(compile_one, SOURCES))
+    for _, warn in results:
+        # hipcc's host pass does not know the device-only feature name: not a problem
+        warn = "\n".join(l for l in warn.splitlines() if "packed-fp32-ops" not in l)
+        if verbose and warn.strip():
+            sys.stderr.write(warn + "\n")
+    objs = [o for o, _ in results]
+    tmp = LIB_PATH + ".tmp"
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs])
+    os.replace(tmp, LIB_PATH)
+    if verbose:
+        print(f"built {LIB_PATH} ({os.path.getsize(LIB_PATH)} bytes)")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build_library()

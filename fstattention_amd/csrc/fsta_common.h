@@ -1,0 +1,61 @@
+// Shared declarations of libfsta's translation units (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "../../include/fsta.h"
+
+namespace fsta {
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// Argument block of every attention kernel.  Plain data, passed by value.
+struct AttnParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    void* o;
+    float* lse;                   // may be null
+    const int64_t* ancestor_idx;  // [nb, max_anc]
+    const uint32_t* mask_bits;    // [nb, mask_words, block_m]
+    const int32_t* anc_count;     // [nb]
+    const int64_t* leaf_idx;      // [nb, block_m]
+    int32_t nq, nk, prefix;       // prefix = nk - nq
+    int32_t block_m, max_anc, mask_words, nb;
+    int32_t heads_total;          // batch * heads
+    int32_t out_f32;              // o is float32 instead of the input type
+    float scale_log2e;            // sm_scale * log2(e)
+};
+
+// Records a message for fsta_last_error() and returns `code`.
+int fail(int code, const char* fmt, ...);
+
+#define FSTA_HIP_OK(expr)                                                          \
+    do {                                                                           \
+        hipError_t err__ = (expr);                                                 \
+        if (err__ != hipSuccess)                                                   \
+            return ::fsta::fail(FSTA_EHIP, "%s: %s", #expr, hipGetErrorString(err__)); \
+    } while (0)
+
+// launchers, one per translation unit
+int launch_attention_generic(const AttnParams& p, int dtype, int head_dim, hipStream_t stream);
+int launch_attention_mfma(const AttnParams& p, int dtype, int head_dim, bool fast_pv,
+                          hipStream_t stream);
+bool mfma_supported(int dtype, int head_dim, int block_m);
+
+// ---- element conversion -------------------------------------------------
+__device__ __forceinline__ float to_float(float x) { return x; }
+__device__ __forceinline__ float to_float(__half x) { return __half2float(x); }
+__device__ __forceinline__ float to_float(__hip_bfloat16 x) { return __bfloat162float(x); }
+
+template <typename T> __device__ __forceinline__ T from_float(float x);
+template <> __device__ __forceinline__ float from_float<float>(float x) { return x; }
+template <> __device__ __forceinline__ __half from_float<__half>(float x) { return __float2half_rn(x); }
+template <> __device__ __forceinline__ __hip_bfloat16 from_float<__hip_bfloat16>(float x) {
+    return __float2bfloat16(x);
+}
+
+}  // namespace fsta

@@ -1,0 +1,119 @@
+"""Block precompute on the GPU: ``create_fst_attention_kernel_inputs``.
+
+Same signature and results as reference ``utils.py:104-129``; the per-block
+Python loop is replaced by one launch of an integer HIP kernel, so a tree that
+changes every decoding step can be re-chunked without leaving the device.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib
+from .attention import PackedTreeMask, _stream_ptr
+
+
+def _raise_for_status(status: int, max_ancestors: int):
+    if status & _lib.PRE_BAD_NODE_ID:
+        raise ValueError("lineage holds a node id outside [-1, n_nodes)")
+    if status & _lib.PRE_BAD_LEVEL:
+        raise IndexError("level_lookup holds a level outside lineage's columns")
+    if status & _lib.PRE_TOO_MANY_ANCESTORS:
+        # the reference fails here with a shape-mismatch RuntimeError (utils.py:120)
+        raise RuntimeError(f"a block has more than max_ancestors={max_ancestors} unique ancestors")
+
+
+def create_fst_attention_kernel_inputs(lineage, level_lookup, block_m=64, max_ancestors=32, *,
+                                       mutate_lineage: bool = True, check: bool = True,
+                                       want_bool_mask: bool = True, device=None):
+    """``(ancestor_idx, ancestor_mask, leaf_idx)`` of reference ``utils.py:104-129``.
+
+    ``ancestor_idx`` int64 ``[NB, max_ancestors]`` (ascending, ``-1`` padded),
+    ``ancestor_mask`` bool ``[NB, block_m, max_ancestors]``, ``leaf_idx`` int64
+    ``[NB, block_m]``, on the device of ``lineage``.  CPU inputs are staged
+    through the GPU (``device`` or the current one) and come back as CPU tensors;
+    GPU inputs stay there, and the returned ``ancestor_mask`` carries its packed
+    form so ``fst_attention`` does not repack it.  Like the reference the
+    caller's ``lineage`` receives each node's id in its own level column unless
+    ``mutate_lineage=False``.  ``check`` synchronises to raise the reference's
+    ``RuntimeError`` when a block has more than ``max_ancestors`` ancestors;
+    with ``check=False`` a 4th value, the device status word, is returned
+    instead.  ``want_bool_mask=False`` returns a :class:`PackedTreeMask` in
+    place of the bool tensor.
+    """
+    if lineage.dim() != 2 or level_lookup.dim() != 1 or level_lookup.shape[0] != lineage.shape[0]:
+        raise ValueError(f"lineage {tuple(lineage.shape)} / level_lookup {tuple(level_lookup.shape)}")
+    if lineage.dtype != torch.int64 or level_lookup.dtype != torch.int64:
+        raise ValueError("lineage and level_lookup must be int64")
+    block_m = int(block_m)
+    max_ancestors = int(max_ancestors)
+    lib = _lib.load()
+    on_host = not lineage.is_cuda
+    if on_host:
+        if not torch.cuda.is_available():
+            raise RuntimeError("create_fst_attention_kernel_inputs runs on the GPU only "
+                               "(no CPU fallback) and no GPU is available")
+        dev = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())
+    else:
+        dev = lineage.device
+    lin = lineage.to(dev).contiguous()
+    lvl = level_lookup.to(dev).contiguous()
+    n, width = lin.shape
+    nb = -(-n // block_m)
+    words = (max_ancestors + 31) // 32
+    a_idx = torch.empty((nb, max_ancestors), dtype=torch.int64, device=dev)
+    a_mask = torch.empty((nb, block_m, max_ancestors), dtype=torch.bool, device=dev) if want_bool_mask else None
+    l_idx = torch.empty((nb, block_m), dtype=torch.int64, device=dev)
+    bits = torch.empty((nb, words, block_m), dtype=torch.int32, device=dev)
+    count = torch.empty((nb,), dtype=torch.int32, device=dev)
+    status = torch.zeros((1,), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(lib.fsta_precompute(
+            lin.data_ptr(), lvl.data_ptr(), n, width, block_m, max_ancestors, int(mutate_lineage),
+            a_idx.data_ptr(), a_mask.data_ptr() if want_bool_mask else None, l_idx.data_ptr(),
+            bits.data_ptr(), count.data_ptr(), status.data_ptr(), _stream_ptr(dev)))
+    if check:
+        _raise_for_status(int(status.item()), max_ancestors)
+    if mutate_lineage and lin.data_ptr() != lineage.data_ptr():
+        lineage.copy_(lin)
+    packed = PackedTreeMask(bits, count, block_m, max_ancestors)
+    if on_host:
+        out = (a_idx.cpu(), a_mask.cpu() if want_bool_mask else packed, l_idx.cpu())
+    else:
+        if want_bool_mask:
+            key = (a_mask._version, a_idx.data_ptr(), a_idx._version, tuple(a_mask.shape))
+            a_mask._fsta_packed = (key, packed)
+        out = (a_idx, a_mask if want_bool_mask else packed, l_idx)
+    return out if check else out + (status,)
+
+
+def lineage_from_parents_gpu(parent: torch.Tensor, width: Optional[int] = None, check: bool = True):
+    """``parent [N]`` int64 on the GPU -> ``(lineage [N, width], level_lookup [N])`` on the GPU.
+
+    Layout of reference ``utils.py:66-75``.  Without ``width`` the levels are
+    computed first and ``max(level) + 1`` is read back (one synchronisation).
+    """
+    if not parent.is_cuda or parent.dtype != torch.int64 or parent.dim() != 1:
+        raise ValueError("parent must be a 1-D int64 tensor on the GPU")
+    lib = _lib.load()
+    parent = parent.contiguous()
+    dev = parent.device
+    n = parent.shape[0]
+    level = torch.empty((n,), dtype=torch.int64, device=dev)
+    status = torch.zeros((1,), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        if width is None:
+            _lib.check(lib.fsta_lineage_from_parents(parent.data_ptr(), n, 1, None, level.data_ptr(),
+                                                     status.data_ptr(), _stream_ptr(dev)))
+            width = int(level.max().item()) + 1 if n else 1
+        lineage = torch.empty((n, width), dtype=torch.int64, device=dev)
+        _lib.check(lib.fsta_lineage_from_parents(parent.data_ptr(), n, width, lineage.data_ptr(),
+                                                 level.data_ptr(), status.data_ptr(), _stream_ptr(dev)))
+    if check:
+        st = int(status.item())
+        if st & _lib.PRE_BAD_NODE_ID:
+            raise ValueError("parent[i] must lie in [-1, i)")
+        if st & _lib.PRE_BAD_LEVEL:
+            raise ValueError(f"tree is deeper than width={width}")
+    return lineage, level

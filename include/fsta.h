@@ -1,0 +1,136 @@
+/*
+ * fsta.h -- C ABI of libfsta: fused sparse tree attention for AMD MI355X (gfx950).
+ *
+ * Every pointer is a DEVICE pointer unless its comment says "host".  `stream`
+ * is a hipStream_t passed as void* (NULL = the null stream).  All entry points
+ * only enqueue work on `stream`; none synchronises, allocates or frees memory.
+ * Return value: FSTA_OK or a negative FSTA_E* code; fsta_last_error() then
+ * gives a message for the calling thread.
+ *
+ * Tensors are dense row-major ("contiguous") with the shapes given below.
+ * Conventions shared with the reference: node ids are int64, -1 marks an empty
+ * slot, ancestor_mask is one byte per entry (0/1).
+ */
+#ifndef FSTA_H
+#define FSTA_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FSTA_ABI_VERSION 1
+
+/* element types of q/k/v/o */
+#define FSTA_F32  0
+#define FSTA_F16  1
+#define FSTA_BF16 2
+
+/* return codes */
+#define FSTA_OK            0
+#define FSTA_EINVAL       -1  /* argument outside the documented domain      */
+#define FSTA_EUNSUPPORTED -2  /* valid but not built (head_dim, block size)   */
+#define FSTA_EHIP         -3  /* the HIP runtime reported an error            */
+
+/* flags of fsta_attention_fwd */
+#define FSTA_FLAG_FAST_PV   1u /* bf16 only: feed P to the matrix cores as one bf16
+                                  value instead of a hi+lo pair (about 2^-9 relative
+                                  error per weight instead of 2^-17)            */
+#define FSTA_FLAG_GENERIC   2u /* force the scalar-ALU kernel (any dtype)      */
+
+/* bits of the status word written by fsta_precompute */
+#define FSTA_PRE_TOO_MANY_ANCESTORS 1u /* a block has more than max_ancestors unique ancestors */
+#define FSTA_PRE_BAD_NODE_ID        2u /* lineage entry < -1 or >= n_nodes                      */
+#define FSTA_PRE_BAD_LEVEL          4u /* level_lookup entry outside [-width, width)            */
+
+int fsta_abi_version(void);
+
+/* Message of the last failing call made by this thread ("" if none). */
+const char* fsta_last_error(void);
+
+/* Number of 32-bit words per (block, query row) in the packed tree mask. */
+int32_t fsta_mask_words(int32_t max_ancestors);
+
+/*
+ * Per-block tree precompute on the GPU; replaces the host loop of
+ * create_fst_attention_kernel_inputs (reference utils.py:104-129) and is
+ * bit-exact with it:
+ *   ancestor_idx  [num_blocks, max_ancestors]           int64  (utils.py:112,119-120)
+ *   ancestor_mask [num_blocks, block_m, max_ancestors]  bool   (utils.py:113,126-127)
+ *   leaf_idx      [num_blocks, block_m]                 int64  (utils.py:114,121-122)
+ * with num_blocks = ceil(n_nodes / block_m); ancestor_mask may be NULL when only
+ * the packed form is wanted.  Extra outputs for the attention kernel (either
+ * may be NULL):
+ *   mask_bits     [num_blocks, fsta_mask_words(A), block_m] uint32, bit b of
+ *                 word w of row r = ancestor_mask[j, r, 32*w + b]
+ *   anc_count     [num_blocks] int32, number of valid entries of ancestor_idx[j]
+ * lineage [n_nodes, width] int64 and level_lookup [n_nodes] int64 follow the
+ * layout of utils.py:43-44,66-75.  With mutate_lineage != 0 each node id is
+ * written into its own level column of `lineage`, as utils.py:124-125 does to
+ * the caller's tensor.  `status` (one uint32, must be zero on entry) receives
+ * FSTA_PRE_* bits; where the reference raises (utils.py:120) the bit
+ * FSTA_PRE_TOO_MANY_ANCESTORS is set and the surplus ancestors are dropped.
+ */
+int fsta_precompute(int64_t* lineage, const int64_t* level_lookup,
+                    int64_t n_nodes, int64_t width,
+                    int32_t block_m, int32_t max_ancestors, int32_t mutate_lineage,
+                    int64_t* ancestor_idx, uint8_t* ancestor_mask, int64_t* leaf_idx,
+                    uint32_t* mask_bits, int32_t* anc_count, uint32_t* status,
+                    void* stream);
+
+/*
+ * Packs a boolean ancestor_mask [num_blocks, block_m, max_ancestors] (one byte
+ * per entry, the tensor utils.py:104-129 returns) into mask_bits (layout above)
+ * and counts, per block, the leading slots of ancestor_idx up to and including
+ * the last non-negative one into anc_count.  Bits of slots whose ancestor_idx
+ * is negative are cleared.
+ */
+int fsta_pack_mask(const int64_t* ancestor_idx, const uint8_t* ancestor_mask,
+                   int32_t num_blocks, int32_t block_m, int32_t max_ancestors,
+                   uint32_t* mask_bits, int32_t* anc_count, void* stream);
+
+/*
+ * Fused sparse tree attention forward; replaces fst_attention/_fwd_kernel
+ * (reference fstattention.py:153-181, 21-151).
+ *   q [batch, heads, nq, head_dim], k, v [batch, heads, nk, head_dim] of `dtype`;
+ *   o [batch, heads, nq, head_dim] of `out_dtype` (= dtype, or FSTA_F32);
+ *   lse [batch*heads, nq] float32 or NULL: base-2 log-sum-exp of the scaled
+ *   scores times log2(e) (fstattention.py:139-141).
+ * Query block j = rows [j*block_m, (j+1)*block_m) attends, per row r, to
+ *   - K/V rows ancestor_idx[j, c] for the columns c whose mask bit is set,
+ *   - K/V row leaf_idx[j, r] if that is >= 0 (fstattention.py:86-91,104-107),
+ *   - K/V rows [0, nk - nq), the shared dense prefix (fstattention.py:113-136),
+ * with weights softmax(q.k * sm_scale) over that set.  Negative indices and
+ * indices >= nk are skipped.  nq need not be a multiple of block_m (the rows
+ * past nq are neither read nor written) and the prefix may have any length;
+ * num_blocks must equal ceil(nq / block_m).  A row that attends to nothing
+ * gets o = 0 and lse = -inf.
+ * head_dim in {16,32,64,128}; block_m in {16,32,64,128}; max_ancestors >= 1.
+ */
+int fsta_attention_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
+                       const int64_t* ancestor_idx, const uint32_t* mask_bits,
+                       const int32_t* anc_count, const int64_t* leaf_idx,
+                       int32_t batch, int32_t heads, int32_t nq, int32_t nk, int32_t head_dim,
+                       int32_t dtype, int32_t out_dtype,
+                       int32_t block_m, int32_t max_ancestors, int32_t num_blocks,
+                       float sm_scale, uint32_t flags, void* stream);
+
+/*
+ * parent[n_nodes] int64 (parent[i] < i, -1 for roots) -> level_lookup [n_nodes]
+ * and lineage [n_nodes, width] in the layout of utils.py:66-75 (strict ancestor
+ * a of i at lineage[i, level(a)], -1 elsewhere).  `status` (zero on entry) gets
+ * FSTA_PRE_BAD_NODE_ID for an entry outside [-1, i) and FSTA_PRE_BAD_LEVEL when
+ * a node is deeper than width-1.  With lineage == NULL only level_lookup is
+ * written (to size `width` first).  Front-end for trees that are rebuilt on the
+ * GPU every decoding step; the reference builds lineage on the host only
+ * (utils.py:66-75).
+ */
+int fsta_lineage_from_parents(const int64_t* parent, int64_t n_nodes, int64_t width,
+                              int64_t* lineage, int64_t* level_lookup, uint32_t* status,
+                              void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FSTA_H */

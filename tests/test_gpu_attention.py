@@ -1,0 +1,238 @@
+"""GPU parity of the fused sparse tree attention against the dense-masked oracle.
+
+Tolerances: float32 atol=rtol=1e-5; float16/bfloat16 atol=rtol=2e-3 against the
+float64 oracle evaluated on the same (already rounded) inputs, asserted on the
+float32 output of the kernel.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from fstattention_amd import (create_fst_attention_kernel_inputs, fst_attention, shift_for_prefix,
+                              trees)
+from helpers import TOL, assert_close, dense_oracle, oracle_inputs, rand_qkv
+from oracle import tree_precompute as tp
+
+pytestmark = pytest.mark.gpu
+
+
+def run_tree(parent, block_m, z, h, d, dtype, seed, prefix=0, generic=False, fast_pv=False,
+             scale=None, check_lse=True):
+    n = len(parent)
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(parent, block_m)
+    nb = a_idx.shape[0]
+    nq = nb * block_m            # the reference needs whole blocks; pad rows see themselves
+    q, k, v = rand_qkv(z, h, nq, nq + prefix, d, dtype, seed)
+    scale = scale if scale is not None else 1.0 / math.sqrt(d)
+    want, want_lse = dense_oracle(q, k, v, parent, scale, prefix=prefix, nq_pad=nq - n)
+    if prefix:
+        a_idx, l_idx = shift_for_prefix(a_idx, l_idx, prefix)
+    o, lse = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(),
+                           scale, BLOCK_M=block_m, MAX_ANCESTORS=max_anc,
+                           out_dtype=torch.float32, return_lse=True, generic=generic, fast_pv=fast_pv)
+    assert o.dtype == torch.float32 and o.shape == q.shape
+    err = assert_close(o, want, dtype, f"n={n} m={block_m} d={d} {dtype} prefix={prefix}")
+    if check_lse:
+        lse_tol = 1e-4 if dtype == torch.float32 else 2e-3
+        torch.testing.assert_close(lse.cpu().double().view(z, h, nq), want_lse, atol=lse_tol, rtol=lse_tol)
+    return err
+
+
+@pytest.mark.parametrize("generic", [False, True])
+def test_config1_random64_fp32(generic):
+    cfg = trees.config(1)
+    run_tree(cfg.parent, cfg.block_m, cfg.batch, cfg.heads, cfg.head_dim, torch.float32,
+             cfg.tensor_seed, generic=generic)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("generic", [False, True])
+def test_config2_medusa256(dtype, generic):
+    cfg = trees.config(2)
+    run_tree(cfg.parent, cfg.block_m, cfg.batch, cfg.heads, cfg.head_dim, dtype, cfg.tensor_seed,
+             generic=generic)
+
+
+@pytest.mark.parametrize("index", [3, 4])
+def test_config3_4_bf16(index):
+    cfg = trees.config(index)
+    run_tree(cfg.parent, cfg.block_m, cfg.batch, cfg.heads, cfg.head_dim, torch.bfloat16,
+             cfg.tensor_seed)
+
+
+def test_config5_bf16_head_subset_against_oracle():
+    # full tree and block size, 8 of the 512 (batch, head) slices so the oracle stays small
+    cfg = trees.config(5)
+    run_tree(cfg.parent, cfg.block_m, 2, 4, cfg.head_dim, torch.bfloat16, cfg.tensor_seed)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("d", [16, 32, 64, 128])
+@pytest.mark.parametrize("block_m", [16, 32, 64, 128])
+def test_shapes_sweep(dtype, d, block_m):
+    parent = trees.random_recursive_parents(200, 100 + d + block_m, window=48)
+    run_tree(parent, block_m, 1, 3, d, dtype, 7)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("prefix", [64, 100, 7])
+def test_shared_prefix(dtype, prefix):
+    parent = trees.random_recursive_parents(128, 5, window=32)
+    run_tree(parent, 64, 2, 2, 64, dtype, 11, prefix=prefix)
+
+
+def test_reference_test_shape_with_and_without_prefix():
+    # the reference's own test: Z=2 H=2 N_CTX=2048 D=64 fp16, tree of 2044 nodes,
+    # blocks of 128, 64 ancestors, sm_scale 0.5, inputs N(0, 0.5^2), prefix 0 or 2048
+    lineage, level = trees.create_tree(trees.DEPTH_MAPPING[2048])
+    parent = trees.parents_from_lineage(lineage, level)
+    a_idx, a_mask, l_idx = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), 128,
+                                                              trees.MAX_ANCESTOR_MAPPING[2048])
+    for prefix in (0, 2048):
+        q, k, v = rand_qkv(2, 2, 2048, 2048 + prefix, 64, torch.float16, 20)
+        q, k, v = q * 0.5, k * 0.5, v * 0.5
+        want, _ = dense_oracle(q, k, v, parent, 0.5, prefix=prefix, nq_pad=4)
+        ai, li = shift_for_prefix(a_idx, l_idx, prefix) if prefix else (a_idx, l_idx)
+        o = fst_attention(q.cuda(), k.cuda(), v.cuda(), ai, a_mask, li, 0.5)   # defaults 128 / 64
+        assert o.dtype == torch.float16
+        # the reference's own criterion on its own output dtype
+        assert torch.allclose(o.cpu().float(), want.float(), atol=1e-2, rtol=0)
+        o32 = fst_attention(q.cuda(), k.cuda(), v.cuda(), ai, a_mask, li, 0.5, out_dtype=torch.float32)
+        assert_close(o32, want, torch.float16, f"reference shape prefix={prefix}")
+
+
+def test_ragged_query_count():
+    # nq not a multiple of block_m: rows past nq are neither read nor written
+    parent = trees.random_recursive_parents(100, 3)
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(parent, 32)
+    for dtype in (torch.float32, torch.bfloat16):
+        q, k, v = rand_qkv(1, 2, 100, 100, 64, dtype, 5)
+        want, _ = dense_oracle(q, k, v, parent, 0.125)
+        o = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(),
+                          0.125, BLOCK_M=32, MAX_ANCESTORS=max_anc, out_dtype=torch.float32)
+        assert_close(o, want, dtype, "ragged")
+
+
+def test_closed_forms_roots_and_equal_keys():
+    parent = np.array([-1, -1, 0, 1, -1, 2, 5, 6] + [7] * 8)
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(parent, 16)
+    q, k, v = rand_qkv(1, 2, 16, 16, 32, torch.float16, 9)
+    args = (a_idx.cuda(), a_mask.cuda(), l_idx.cuda(), 0.3)
+    o = fst_attention(q.cuda(), k.cuda(), v.cuda(), *args, BLOCK_M=16, MAX_ANCESTORS=max_anc)
+    for r in (0, 1, 4):    # roots attend to themselves only: o = v exactly
+        assert torch.equal(o[0, :, r].cpu(), v[0, :, r])
+    k_same = k[:, :, :1].expand_as(k).contiguous()
+    o = fst_attention(q.cuda(), k_same.cuda(), v.cuda(), *args, BLOCK_M=16, MAX_ANCESTORS=max_anc,
+                      out_dtype=torch.float32)
+    m = torch.from_numpy(tp.dense_tree_mask(parent)).double()
+    want = (m @ v.double()) / m.sum(-1, keepdim=True)
+    assert_close(o, want, torch.float16, "equal keys -> mean of allowed values")
+
+
+def test_default_output_dtype_and_bf16_rounding_report():
+    cfg = trees.config(2)
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(cfg.parent, cfg.block_m)
+    q, k, v = trees.make_qkv(cfg)
+    scale = 1 / math.sqrt(cfg.head_dim)
+    want, _ = dense_oracle(q, k, v, cfg.parent, scale)
+    o = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(), scale,
+                      BLOCK_M=cfg.block_m, MAX_ANCESTORS=max_anc)
+    assert o.dtype == torch.bfloat16
+    # a bf16 result can be no closer than the oracle rounded to bf16: at most one ulp apart
+    # (plus the float32 accumulation error, which matters only where values cancel to ~0)
+    ulp = torch.maximum(want.abs(), torch.tensor(2.0 ** -126)).log2().floor().exp2() * 2.0 ** -7
+    assert ((o.cpu().double() - want).abs() <= ulp + 1e-6).all()
+
+
+def test_fast_pv_flag_stays_within_loose_bound():
+    cfg = trees.config(2)
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(cfg.parent, cfg.block_m)
+    q, k, v = trees.make_qkv(cfg)
+    scale = 1 / math.sqrt(cfg.head_dim)
+    want, _ = dense_oracle(q, k, v, cfg.parent, scale)
+    o = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(), scale,
+                      BLOCK_M=cfg.block_m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32, fast_pv=True)
+    assert (o.cpu().double() - want).abs().max() < 1e-2
+
+
+def test_ancestor_slots_with_holes_and_out_of_range_ids_are_skipped():
+    parent = trees.random_recursive_parents(64, 8)
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(parent, 32, multiple=8)
+    # widen the ancestor axis and move the valid entries to odd slots; fill even slots with
+    # -1 or ids past the end of K whose mask bits are set: they must be ignored
+    nb = a_idx.shape[0]
+    wide_idx = torch.full((nb, 2 * max_anc), -1, dtype=torch.int64)
+    wide_mask = torch.zeros((nb, 32, 2 * max_anc), dtype=torch.bool)
+    wide_idx[:, 1::2] = a_idx
+    wide_mask[:, :, 1::2] = a_mask
+    wide_idx[:, 0::4] = 10 ** 6
+    wide_mask[:, :, 0::2] = True
+    q, k, v = rand_qkv(1, 2, 64, 64, 64, torch.float32, 3)
+    want, _ = dense_oracle(q, k, v, parent, 0.2)
+    for generic in (False, True):
+        o = fst_attention(q.cuda(), k.cuda(), v.cuda(), wide_idx.cuda(), wide_mask.cuda(), l_idx.cuda(),
+                          0.2, BLOCK_M=32, MAX_ANCESTORS=2 * max_anc, generic=generic)
+        assert_close(o, want, torch.float32, "holes")
+
+
+def test_rows_without_any_key_give_zero():
+    a_idx = torch.full((1, 8), -1, dtype=torch.int64)
+    a_mask = torch.zeros((1, 16, 8), dtype=torch.bool)
+    l_idx = torch.full((1, 16), -1, dtype=torch.int64)
+    l_idx[0, 3] = 3
+    q, k, v = rand_qkv(1, 1, 16, 16, 16, torch.float16, 1)
+    o, lse = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(), 1.0,
+                           BLOCK_M=16, MAX_ANCESTORS=8, return_lse=True)
+    assert torch.equal(o[0, 0, 3].cpu(), v[0, 0, 3])
+    rest = [r for r in range(16) if r != 3]
+    assert (o[0, 0, rest] == 0).all() and torch.isinf(lse[0, rest]).all()
+
+
+def test_argument_errors():
+    q, k, v = (t.cuda() for t in rand_qkv(1, 1, 16, 16, 16, torch.float16, 1))
+    a_idx = torch.full((1, 8), -1, dtype=torch.int64).cuda()
+    a_mask = torch.zeros((1, 16, 8), dtype=torch.bool).cuda()
+    l_idx = torch.arange(16).view(1, 16).cuda()
+    fst_attention(q, k, v, a_idx, a_mask, l_idx, 1.0, BLOCK_M=16, MAX_ANCESTORS=8)
+    with pytest.raises(AssertionError):     # the reference's assertion on the head dimension
+        fst_attention(q[..., :8].contiguous(), k[..., :8].contiguous(), v[..., :8].contiguous(),
+                      a_idx, a_mask, l_idx, 1.0, BLOCK_M=16, MAX_ANCESTORS=8)
+    with pytest.raises(AssertionError):
+        fst_attention(q, k, v[..., :8].contiguous(), a_idx, a_mask, l_idx, 1.0, BLOCK_M=16, MAX_ANCESTORS=8)
+    with pytest.raises(ValueError):         # defaults 128 / 64 do not match these tensors
+        fst_attention(q, k, v, a_idx, a_mask, l_idx, 1.0)
+    with pytest.raises(ValueError):
+        fst_attention(q.transpose(1, 2), k, v, a_idx, a_mask, l_idx, 1.0, BLOCK_M=16, MAX_ANCESTORS=8)
+    with pytest.raises(ValueError):
+        fst_attention(q.cpu(), k.cpu(), v.cpu(), a_idx, a_mask, l_idx, 1.0, BLOCK_M=16, MAX_ANCESTORS=8)
+    with pytest.raises(ValueError):
+        fst_attention(q, k.float(), v, a_idx, a_mask, l_idx, 1.0, BLOCK_M=16, MAX_ANCESTORS=8)
+
+
+def test_mask_cache_follows_in_place_edits():
+    parent = trees.random_recursive_parents(32, 4)
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(parent, 32)
+    q, k, v = (t.cuda() for t in rand_qkv(1, 1, 32, 32, 32, torch.float32, 2))
+    a_idx, a_mask, l_idx = a_idx.cuda(), a_mask.cuda(), l_idx.cuda()
+    o1 = fst_attention(q, k, v, a_idx, a_mask, l_idx, 0.2, BLOCK_M=32, MAX_ANCESTORS=max_anc)
+    a_mask.zero_()                      # now every row only sees itself if it is a leaf
+    o2 = fst_attention(q, k, v, a_idx, a_mask, l_idx, 0.2, BLOCK_M=32, MAX_ANCESTORS=max_anc)
+    leaf_rows = (l_idx[0] >= 0).nonzero().flatten()
+    assert torch.equal(o2[0, 0, leaf_rows], v[0, 0, leaf_rows])
+    assert not torch.equal(o1, o2)
+
+
+def test_non_default_stream():
+    cfg = trees.config(1)
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(cfg.parent, cfg.block_m)
+    q, k, v = trees.make_qkv(cfg)
+    want, _ = dense_oracle(q, k, v, cfg.parent, 0.125)
+    dev = [t.cuda() for t in (q, k, v, a_idx, a_mask, l_idx)]
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        o = fst_attention(*dev, 0.125, BLOCK_M=cfg.block_m, MAX_ANCESTORS=max_anc)
+    s.synchronize()
+    assert_close(o, want, torch.float32, "side stream")

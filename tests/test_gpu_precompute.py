@@ -1,0 +1,146 @@
+"""GPU parity of the integer precompute kernels (bit-exact), through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import golden_cases
+from fstattention_amd import (create_fst_attention_kernel_inputs, lineage_from_parents_gpu,
+                              pack_tree_mask, trees)
+from oracle import tree_precompute as tp
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(got, want):
+    a_idx, a_mask, l_idx = got
+    assert a_idx.dtype == torch.int64 and l_idx.dtype == torch.int64 and a_mask.dtype == torch.bool
+    np.testing.assert_array_equal(a_idx.cpu().numpy(), want[0])
+    np.testing.assert_array_equal(a_mask.cpu().numpy(), want[1])
+    np.testing.assert_array_equal(l_idx.cpu().numpy(), want[2])
+
+
+@pytest.mark.parametrize("case", golden_cases())
+def test_reference_vectors_device_tensors(golden, case):
+    lineage = torch.from_numpy(golden[f"{case}/lineage_in"].copy()).cuda()
+    level = torch.from_numpy(golden[f"{case}/level_lookup"]).cuda()
+    block_m, max_anc = (int(x) for x in golden[f"{case}/params"])
+    got = create_fst_attention_kernel_inputs(lineage, level, block_m, max_anc)
+    assert all(t.is_cuda for t in got)
+    _check(got, [golden[f"{case}/{k}"] for k in ("ancestor_idx", "ancestor_mask", "leaf_idx")])
+    np.testing.assert_array_equal(lineage.cpu().numpy(), golden[f"{case}/lineage_out"])
+
+
+def test_reference_vectors_host_tensors_round_trip(golden):
+    case = "create_tree_d5_k4_f0.5_m64_a32"
+    lineage = torch.from_numpy(golden[f"{case}/lineage_in"].copy())
+    level = torch.from_numpy(golden[f"{case}/level_lookup"])
+    got = create_fst_attention_kernel_inputs(lineage, level, 64, 32)
+    assert not any(t.is_cuda for t in got)
+    _check(got, [golden[f"{case}/{k}"] for k in ("ancestor_idx", "ancestor_mask", "leaf_idx")])
+    np.testing.assert_array_equal(lineage.numpy(), golden[f"{case}/lineage_out"])
+    # second flavour: leave the caller's lineage alone
+    lineage2 = torch.from_numpy(golden[f"{case}/lineage_in"].copy())
+    create_fst_attention_kernel_inputs(lineage2, level, 64, 32, mutate_lineage=False)
+    np.testing.assert_array_equal(lineage2.numpy(), golden[f"{case}/lineage_in"])
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_trees_against_oracle(seed):
+    rng = np.random.default_rng(seed)
+    n = int(rng.integers(1, 700))
+    window = [None, 4, 32][seed % 3]
+    block_m = [16, 64, 128, 8][seed % 4]
+    parent = trees.random_recursive_parents(n, seed, window)
+    parent[rng.random(n) < 0.03] = -1
+    lineage, level = trees.lineage_from_parents(parent)
+    max_anc = trees.required_max_ancestors(parent, block_m, [1, 16, 7][seed % 3])
+    lin_cpu = lineage.numpy().copy()
+    want = tp.block_inputs(lin_cpu, level.numpy(), block_m, max_anc)
+    lin_gpu = lineage.clone().cuda()
+    got = create_fst_attention_kernel_inputs(lin_gpu, level.cuda(), block_m, max_anc)
+    _check(got, want)
+    np.testing.assert_array_equal(lin_gpu.cpu().numpy(), lin_cpu)
+
+
+@pytest.mark.parametrize("index", [3, 4, 5])
+def test_benchmark_trees_full_size(index):
+    cfg = trees.config(index)
+    lineage, level = trees.lineage_from_parents(cfg.parent)
+    max_anc = trees.required_max_ancestors(cfg.parent, cfg.block_m, 16)
+    want = tp.block_inputs(lineage.numpy().copy(), level.numpy(), cfg.block_m, max_anc)
+    got = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), cfg.block_m, max_anc)
+    _check(got, want)
+    # size-independent property: the three tensors rebuild the dense ancestor-or-self mask
+    dense = tp.reconstruct_dense_mask(got[0].cpu().numpy(), got[1].cpu().numpy(),
+                                      got[2].cpu().numpy(), cfg.n_nodes)
+    np.testing.assert_array_equal(dense[:, :cfg.n_nodes], tp.dense_tree_mask(cfg.parent))
+
+
+def test_reference_benchmark_tree_largest():
+    # the reference's largest table entry: 2**17 tokens, depth 14, blocks of 128, 64 ancestors
+    lineage, level = trees.create_tree(14)
+    want = tp.block_inputs(lineage.numpy().copy(), level.numpy(), 128, 64)
+    got = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), 128, 64)
+    _check(got, want)
+
+
+def test_too_many_ancestors_raises_like_the_reference():
+    parent = np.arange(-1, 63)
+    lineage, level = trees.lineage_from_parents(parent)
+    with pytest.raises(RuntimeError):
+        create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), 16, 16)
+    out = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), 16, 16, check=False)
+    assert int(out[3].item()) & 1
+
+
+def test_bad_inputs_are_flagged():
+    lineage, level = trees.lineage_from_parents(np.array([-1, 0, 1, 1]))
+    bad = lineage.clone()
+    bad[3, 0] = 9
+    with pytest.raises(ValueError):
+        create_fst_attention_kernel_inputs(bad.cuda(), level.cuda(), 4, 4)
+    with pytest.raises(IndexError):
+        create_fst_attention_kernel_inputs(lineage.cuda(), (level + 7).cuda(), 4, 4)
+    with pytest.raises(ValueError):
+        create_fst_attention_kernel_inputs(lineage.int().cuda(), level.cuda(), 4, 4)
+
+
+def test_block_without_padding_drops_smallest_id():
+    # every row of the block is full: the reference's `[1:]` then drops the smallest node id
+    lineage = torch.tensor([[0, 1], [0, 1]], dtype=torch.int64)
+    level = torch.tensor([1, 1], dtype=torch.int64)
+    want = tp.block_inputs(lineage.numpy().copy(), level.numpy(), 2, 4)
+    got = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), 2, 4)
+    _check(got, want)
+
+
+def test_packed_mask_matches_bool_mask():
+    parent = trees.random_recursive_parents(500, 42, window=40)
+    lineage, level = trees.lineage_from_parents(parent)
+    max_anc = trees.required_max_ancestors(parent, 64, 1)
+    a_idx, a_mask, l_idx = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), 64, max_anc)
+    from_precompute = a_mask._fsta_packed[1]
+    repacked = pack_tree_mask(a_idx, a_mask)
+    assert torch.equal(from_precompute.mask_bits, repacked.mask_bits)
+    assert torch.equal(from_precompute.anc_count, repacked.anc_count)
+    bits = repacked.mask_bits.cpu().numpy().astype(np.uint32)   # [nb, words, m]
+    mask = a_mask.cpu().numpy()
+    for c in range(max_anc):
+        np.testing.assert_array_equal((bits[:, c // 32, :] >> (c % 32)) & 1, mask[:, :, c])
+    np.testing.assert_array_equal(repacked.anc_count.cpu().numpy(), (a_idx.cpu().numpy() >= 0).sum(1))
+
+
+def test_lineage_from_parents_on_gpu():
+    for seed, window in [(1, None), (2, 8), (3, 64)]:
+        parent = trees.random_recursive_parents(777, seed, window)
+        parent[::97] = -1
+        want_lin, want_lvl = trees.lineage_from_parents(parent)
+        lin, lvl = lineage_from_parents_gpu(torch.from_numpy(parent).cuda())
+        assert torch.equal(lin.cpu(), want_lin) and torch.equal(lvl.cpu(), want_lvl)
+        wide, _ = lineage_from_parents_gpu(torch.from_numpy(parent).cuda(), width=want_lin.shape[1] + 3)
+        assert torch.equal(wide.cpu()[:, :want_lin.shape[1]], want_lin)
+        assert (wide.cpu()[:, want_lin.shape[1]:] == -1).all()
+    with pytest.raises(ValueError):
+        lineage_from_parents_gpu(torch.tensor([-1, 0, 5], dtype=torch.int64).cuda())
+    with pytest.raises(ValueError):
+        lineage_from_parents_gpu(torch.tensor([-1, 0, 1, 2], dtype=torch.int64).cuda(), width=2)
