@@ -1,0 +1,347 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused sparse tree attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--extra]
+
+Workload (the configuration the headline metric is quoted on): 256-node
+Medusa-style tree, B=1, H=32, D=128, bf16, query block 64, synthetic CPU-seeded
+N(0,1) q/k/v, sm_scale = 1/sqrt(D).  A step is one call of the attention entry
+point of the C ABI (``fsta_attention_fwd``) with the per-block kernel inputs
+already built (they are built once per decoding step and reused by every layer,
+which is also how the reference's own benchmark times it).
+
+Timed region: exactly K steps, recorded into one HIP graph so that the host's
+launch rate does not hide the kernel, each step on its own q/k/v/o buffer set;
+the sets rotate over more memory than the 256 MB Infinity Cache, so K/V rows come
+from HBM ("cold").  The same loop over one buffer set ("warm": everything cache
+resident) and plain stream launches are reported beside it.
+
+Prints ONE JSON line.  ``value`` = K/V bytes the op loads per step (per head:
+2*D*2 bytes for every valid ancestor slot and every valid leaf slot of every
+block) divided by the wall time per step.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+if REPO not in sys.path:
+    sys.path.insert(0, REPO)
+
+HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+INFINITY_CACHE_BYTES = 256 << 20
+
+# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/): filled in once measured; None until then.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (headline: 2)")
+    ap.add_argument("--extra", action="store_true", help="also time configurations 3, 4 and 5")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-graph", action="store_true", help="time plain stream launches only")
+    return ap.parse_args()
+
+
+class Workload:
+    """Device-resident inputs of one configuration, in `sets` rotating copies."""
+
+    def __init__(self, index, sets_bytes, dtype=None, heads=None, batch=None):
+        import torch
+        from fstattention_amd import _lib, create_fst_attention_kernel_inputs, trees
+        from fstattention_amd.attention import _DTYPES, _packed_for
+
+        self.torch = torch
+        self.cfg = cfg = trees.config(index, dtype)
+        self.lib = _lib.load()
+        self._check = _lib.check
+        dev = torch.device("cuda", 0)
+        self.z = batch or cfg.batch
+        self.h = heads or cfg.heads
+        self.n, self.d, self.m = cfg.n_nodes, cfg.head_dim, cfg.block_m
+        self.dtype = cfg.dtype
+        self.code = _DTYPES[cfg.dtype]
+        self.esz = torch.tensor([], dtype=cfg.dtype).element_size()
+        self.scale = 1.0 / math.sqrt(self.d)
+
+        # kernel inputs: GPU precompute from the device-resident lineage
+        lineage, level = trees.lineage_from_parents(cfg.parent)
+        self.lineage, self.level = lineage.to(dev), level.to(dev)
+        self.max_anc = trees.required_max_ancestors(cfg.parent, self.m, 16)
+        self.a_idx, self.a_mask, self.l_idx = create_fst_attention_kernel_inputs(
+            self.lineage, self.level, self.m, self.max_anc, mutate_lineage=False)
+        self.packed = _packed_for(self.a_idx, self.a_mask)
+        self.nb = self.a_idx.shape[0]
+        rows = int((self.a_idx >= 0).sum().item() + (self.l_idx >= 0).sum().item())
+        self.kv_rows = rows
+        self.kv_bytes = self.z * self.h * 2 * self.d * self.esz * rows
+        depth = trees.levels_from_parents(cfg.parent)
+        self.pairs = int(depth.sum() + self.n)
+        self.flops = 4 * self.d * self.z * self.h * self.pairs
+
+        per_set = 4 * self.z * self.h * self.n * self.d * self.esz
+        self.per_set_bytes = per_set
+        self.n_sets = max(2, min(256, -(-sets_bytes // per_set)))
+        shape = (self.z, self.h, self.n, self.d)
+        g = torch.Generator().manual_seed(cfg.tensor_seed)
+        self.sets = []
+        base = None
+        for s in range(self.n_sets):
+            if s < 4 or base is None:
+                # CPU-seeded N(0,1), rounded to the storage type, then moved
+                q, k, v = (torch.randn(shape, generator=g, dtype=torch.float32).to(cfg.dtype).to(dev)
+                           for _ in range(3))
+                base = (q, k, v)
+            else:
+                # further sets: device-side copies rolled along the sequence axis (distinct
+                # memory, same distribution) so that building them stays cheap
+                q, k, v = (torch.roll(t, shifts=s, dims=2).contiguous() for t in base)
+            o = torch.empty(shape, dtype=cfg.dtype, device=dev)
+            self.sets.append((q, k, v, o))
+        self.lse = torch.empty((self.z * self.h, self.n), dtype=torch.float32, device=dev)
+
+    def launch(self, s=0, flags=0):
+        """One step: a single call through the C ABI on torch's current stream."""
+        torch = self.torch
+        q, k, v, o = self.sets[s % self.n_sets]
+        self._check(self.lib.fsta_attention_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), self.lse.data_ptr(),
+            self.a_idx.data_ptr(), self.packed.mask_bits.data_ptr(), self.packed.anc_count.data_ptr(),
+            self.l_idx.data_ptr(), self.z, self.h, self.n, self.n, self.d, self.code, self.code,
+            self.m, self.max_anc, self.nb, self.scale, flags, torch.cuda.current_stream().cuda_stream))
+
+    def check_parity(self, heads=2):
+        """Kernel vs CPU oracle on set 0 (first `heads` slices); float32 output, 2e-3 / 1e-5."""
+        torch = self.torch
+        from fstattention_amd import fst_attention
+        from oracle import dense_attention, tree_precompute
+        q, k, v, _ = self.sets[0]
+        hh = min(heads, self.h)
+        qs, ks, vs = (t[:1, :hh].contiguous() for t in (q, k, v))
+        o = fst_attention(qs, ks, vs, self.a_idx, self.a_mask, self.l_idx, self.scale,
+                          BLOCK_M=self.m, MAX_ANCESTORS=self.max_anc, out_dtype=torch.float32)
+        ref, _ = dense_attention.dense_tree_attention(
+            qs.cpu(), ks.cpu(), vs.cpu(), tree_precompute.dense_tree_mask(self.cfg.parent), self.scale)
+        tol = 1e-5 if self.dtype == torch.float32 else 2e-3
+        err = (o.cpu().double() - ref).abs()
+        ok = bool((err <= tol + tol * ref.abs()).all())
+        return ok, float(err.max()), tol
+
+
+def time_steps(wl, steps, warmup, rotate, use_graph, flags=0):
+    """(wall seconds per step, event seconds per step) over exactly `steps` steps."""
+    torch = wl.torch
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for i in range(warmup):
+            wl.launch(i if rotate else 0, flags)
+        stream.synchronize()
+        graph = None
+        if use_graph:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for i in range(steps):
+                    wl.launch(i if rotate else 0, flags)
+            graph.replay()          # one untimed replay: uploads the graph
+            stream.synchronize()
+        ev0 = torch.cuda.Event(enable_timing=True)
+        ev1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ev0.record(stream)
+        if graph is not None:
+            graph.replay()
+        else:
+            for i in range(steps):
+                wl.launch(i if rotate else 0, flags)
+        ev1.record(stream)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    return (t1 - t0) / steps, ev0.elapsed_time(ev1) * 1e-3 / steps
+
+
+def time_python_api(wl, steps, warmup):
+    """Seconds per call of the Python entry point (allocates o and lse every call)."""
+    torch = wl.torch
+    from fstattention_amd import fst_attention
+    q, k, v, _ = wl.sets[0]
+    call = lambda: fst_attention(q, k, v, wl.a_idx, wl.a_mask, wl.l_idx, wl.scale,
+                                 BLOCK_M=wl.m, MAX_ANCESTORS=wl.max_anc)
+    for _ in range(warmup):
+        call()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        call()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def time_precompute(wl, reps=50):
+    """Seconds per GPU rebuild of the kernel inputs (packed mask only, no host sync)."""
+    torch = wl.torch
+    from fstattention_amd import create_fst_attention_kernel_inputs
+    call = lambda: create_fst_attention_kernel_inputs(wl.lineage, wl.level, wl.m, wl.max_anc,
+                                                      mutate_lineage=False, check=False,
+                                                      want_bool_mask=False)
+    for _ in range(5):
+        call()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        call()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / reps
+
+
+def cpu_baseline(wl, budget_s=10.0):
+    """The oracle's dense-masked attention (reference fstattention.py:214-219 restated for
+    the CPU, float32 arithmetic on the bf16-rounded inputs) on the host cores."""
+    import torch
+    from oracle import dense_attention, tree_precompute
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16) if "GRAFT_REPO_ROOT" in os.environ else cores
+    torch.set_num_threads(cores)
+    q, k, v, _ = wl.sets[0]
+    heads = min(wl.h, 32)
+    qs, ks, vs = (t[:1, :heads].cpu() for t in (q, k, v))
+    mask = tree_precompute.dense_tree_mask(wl.cfg.parent)
+    run = lambda: dense_attention.dense_tree_attention(qs, ks, vs, mask, wl.scale, dtype=torch.float32)
+    run()
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 200):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    scale_up = (wl.z * wl.h) / heads      # slices not run: time extrapolated linearly
+    per_call = med * scale_up
+    return {
+        "value": round(wl.kv_bytes / per_call / 1e9, 4),
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "us_per_call": round(per_call * 1e6, 1),
+        "sample": (f"dense-masked attention oracle, float32 on {wl.dtype}-rounded inputs, "
+                   f"{heads} of {wl.z * wl.h} (batch, head) slices of the same workload, "
+                   f"median of {len(times)} runs" + (", scaled linearly to all slices" if scale_up != 1 else "")),
+    }
+
+
+def summarize(wl, steps, warmup, use_graph):
+    cold_wall, cold_ev = time_steps(wl, steps, warmup, rotate=True, use_graph=use_graph)
+    warm_wall, warm_ev = time_steps(wl, steps, warmup, rotate=False, use_graph=use_graph)
+    stream_wall, _ = time_steps(wl, steps, warmup, rotate=True, use_graph=False)
+    return {
+        "cold_us": cold_wall * 1e6, "cold_event_us": cold_ev * 1e6,
+        "warm_us": warm_wall * 1e6, "warm_event_us": warm_ev * 1e6,
+        "stream_launch_us": stream_wall * 1e6,
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU (got --gpus {args.gpus}); the op shards over "
+              "batch*heads without communication, see DESIGN.md", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the hot path has no CPU fallback", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    use_graph = not args.no_graph
+
+    wl = Workload(args.config, sets_bytes=2 * INFINITY_CACHE_BYTES)
+    ok, max_err, tol = wl.check_parity()
+    if not ok:
+        print(f"bench.py: parity check failed (max err {max_err:.3e} > {tol})", file=sys.stderr)
+        sys.exit(1)
+
+    t = summarize(wl, args.steps, args.warmup, use_graph)
+    step_s = t["cold_us"] * 1e-6
+    kernel_s = t["cold_event_us"] * 1e-6
+    achieved = wl.kv_bytes / kernel_s / 1e9
+    result = {
+        "metric": "K/V GB/s loaded (us/call in us_per_call), 256-node Medusa tree H32 D128 bf16"
+                  if args.config == 2 else f"K/V GB/s loaded, {wl.cfg.name}",
+        "value": round(wl.kv_bytes / step_s / 1e9, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 6),
+        "us_per_call": round(step_s * 1e6, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[wl.dtype],
+        "data": "synthetic",
+        "config": {
+            "workload": wl.cfg.name, "nodes": wl.n, "batch": wl.z, "heads": wl.h, "head_dim": wl.d,
+            "block_m": wl.m, "max_ancestors": wl.max_anc, "kv_rows_per_head": wl.kv_rows,
+            "kv_bytes_per_call": wl.kv_bytes, "attended_pairs": wl.pairs, "flops_per_call": wl.flops,
+            "timed_region": ("hip graph of K steps" if use_graph else "K stream launches") +
+                            f", {wl.n_sets} rotating q/k/v/o sets ({wl.n_sets * wl.per_set_bytes >> 20} MiB)",
+        },
+        "effective_tflops": round(wl.flops / step_s / 1e12, 4),
+        "parity": {"max_abs_err_vs_oracle": max_err, "tol": tol, "ok": ok},
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "attn_mfma_kernel<bf16, D=128, M=64, split P>" if args.config == 2 else "attn_mfma_kernel",
+            "achieved": round(achieved, 2),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 5),
+            "traffic": MEASURED_TRAFFIC_BYTES if args.config == 2 else None,
+            "algorithmic_bytes_per_launch": wl.kv_bytes,
+            "avg_launch_us": round(kernel_s * 1e6, 3),
+            "mfma_frac_of_bf16_peak": round(wl.flops / kernel_s / 1e12 / MFMA_BF16_PEAK_TFLOPS, 6),
+        },
+        "regimes_us_per_call": {
+            "cold_graph": round(t["cold_us"], 3), "warm_graph": round(t["warm_us"], 3),
+            "cold_stream_launches": round(t["stream_launch_us"], 3),
+            "python_api_warm": round(time_python_api(wl, args.steps, args.warmup) * 1e6, 3),
+            "gpu_precompute": round(time_precompute(wl) * 1e6, 3),
+        },
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(wl)
+    if args.extra:
+        extra = {}
+        for idx in (3, 4, 5):
+            w = Workload(idx, sets_bytes=2 * INFINITY_CACHE_BYTES)
+            ok_i, err_i, _ = w.check_parity()
+            steps = max(20, min(args.steps, 100 if idx == 5 else args.steps))
+            ti = summarize(w, steps, min(args.warmup, 10), use_graph)
+            ks = ti["cold_event_us"] * 1e-6
+            extra[w.cfg.name] = {
+                "us_per_call_cold": round(ti["cold_us"], 2), "us_per_call_warm": round(ti["warm_us"], 2),
+                "kv_bytes_per_call": w.kv_bytes, "kv_gbps_cold": round(w.kv_bytes / ks / 1e9, 1),
+                "hbm_frac": round(w.kv_bytes / ks / 1e9 / HBM_PEAK_GBPS, 4),
+                "effective_tflops": round(w.flops / ks / 1e12, 3),
+                "gpu_precompute_us": round(time_precompute(w) * 1e6, 2),
+                "parity_ok": ok_i, "max_abs_err": err_i,
+                "batch": w.z, "heads": w.h, "max_ancestors": w.max_anc,
+            }
+            del w
+            torch.cuda.empty_cache()
+        result["extra"] = extra
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -141,9 +141,10 @@ def test_default_output_dtype_and_bf16_rounding_report():
                       BLOCK_M=cfg.block_m, MAX_ANCESTORS=max_anc)
     assert o.dtype == torch.bfloat16
     # a bf16 result can be no closer than the oracle rounded to bf16: at most one ulp apart
-    # (plus the float32 accumulation error, which matters only where values cancel to ~0)
+    # (plus the error of the hi+lo bf16 weights, 2^-17 relative per term, which matters only
+    # where the terms cancel to ~0)
     ulp = torch.maximum(want.abs(), torch.tensor(2.0 ** -126)).log2().floor().exp2() * 2.0 ** -7
-    assert ((o.cpu().double() - want).abs() <= ulp + 1e-6).all()
+    assert ((o.cpu().double() - want).abs() <= ulp + 1e-4).all()
 
 
 def test_fast_pv_flag_stays_within_loose_bound():
