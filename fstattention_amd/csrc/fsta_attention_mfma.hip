@@ -3,7 +3,12 @@
 //
 // One workgroup owns one query block of one (batch, head) slice; each of its
 // M/32 waves owns 32 query rows and keeps their state in registers for the whole
-// kernel.  Work per 32-key tile:
+// kernel.  The block's own rows (the "leaf" diagonal of reference
+// fstattention.py:86-91,104-107: one key per query) never go through LDS: every
+// lane dots its Q registers with its own leaf row and seeds the running softmax
+// with it.  All other keys are processed in tiles of 32: first the block's unique
+// ancestors under the packed tree mask, then the dense shared prefix
+// (fstattention.py:113-136).  Work per tile:
 //
 //   S^T[key, q] = K_tile . Q^T        v_mfma_f32_32x32x16, K fragments from LDS,
 //                                     Q fragments loaded once from HBM into VGPRs
@@ -17,55 +22,67 @@
 // B-operand layout of the second product, so P never touches LDS.  For bf16 the
 // weights are fed as a hi+lo pair of bf16 values (two MFMAs) unless
 // FSTA_FLAG_FAST_PV asks for one; fp16 weights are precise enough as they are.
+// The running maximum is only raised when a row's new maximum exceeds it by more
+// than 2^8, so the accumulator rescale is rare; weights stay below 2^8.
 //
 // K/V rows are gathered from HBM straight into LDS (global_load_lds_dwordx4: 16
 // bytes per lane, one row = D*2 bytes = a run of consecutive lanes, no register
-// staging).  LDS holds a ring of STAGES tiles; the gathers of the next STAGES-1
-// tiles are in flight while the current one is multiplied, which is what keeps
-// enough bytes outstanding to use HBM.  The tiles are XOR-swizzled by choosing
-// which 16-byte chunk of its row a lane fetches.  The block's own rows (the
-// "leaf" diagonal of reference fstattention.py:86-91,104-107) never go through
-// LDS: every lane dots its Q registers with its own leaf row and seeds the
-// running softmax with it.
+// staging).  LDS holds a ring of `stages` tiles; the gathers of the next
+// stages-1 tiles are in flight while the current one is multiplied, which is
+// what keeps enough bytes outstanding to use HBM.  The tiles are XOR-swizzled by
+// choosing which 16-byte chunk of its row a lane fetches.
 #include "fsta_common.h"
 
 namespace fsta {
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kTileN = 32;   // keys per tile
-constexpr int kXcds = 8;     // L2 domains of an MI355X; workgroup i runs on XCD i % 8
+constexpr int kTileN = 32;     // keys per tile
+constexpr int kXcds = 8;       // L2 domains of an MI355X; workgroup i runs on XCD i % 8
+constexpr int kMaxStages = 4;  // ring depth limit (LDS per workgroup = stages * 4 * 32 * D bytes)
+constexpr float kRescaleSlack = 8.f;  // log2 of the largest weight kept without raising the maximum
 
 template <bool BF16> struct Mma;
 template <> struct Mma<true> {
     using elem = __bf16;
+    using elem2 = bf16x2;
     using frag = bf16x8;
     static __device__ __forceinline__ f32x16 mfma(frag a, frag b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
-    static __device__ __forceinline__ float to_f32(elem x) { return (float)x; }
+    static __device__ __forceinline__ float dot2(elem2 a, elem2 b, float c) {
+        return __builtin_amdgcn_fdot2_f32_bf16(a, b, c, false);
+    }
 };
 template <> struct Mma<false> {
     using elem = _Float16;
+    using elem2 = f16x2;
     using frag = f16x8;
     static __device__ __forceinline__ f32x16 mfma(frag a, frag b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
     }
-    static __device__ __forceinline__ float to_f32(elem x) { return (float)x; }
+    static __device__ __forceinline__ float dot2(elem2 a, elem2 b, float c) {
+        return __builtin_amdgcn_fdot2(a, b, c, false);
+    }
 };
 
 __host__ __device__ constexpr int anc_tile_capacity(int max_anc) { return (max_anc + kTileN - 1) / kTileN; }
 
-template <int D, int M, int STAGES>
-__host__ __device__ constexpr size_t mfma_lds_bytes(int max_anc) {
-    // ring of K|V tiles, then per ancestor tile: 32 sanitised keys, one validity word, M mask words
-    return (size_t)STAGES * 2 * kTileN * D * 2 + (size_t)anc_tile_capacity(max_anc) * (kTileN * 4 + 4 + M * 4);
+// LDS of one workgroup: ring of K|V tiles, then per ancestor tile 32 sanitised keys,
+// one validity word and M mask words.
+template <int D, int M>
+__host__ __device__ constexpr size_t mfma_lds_bytes(int max_anc, int stages) {
+    return (size_t)stages * 2 * kTileN * D * 2 +
+           (size_t)anc_tile_capacity(max_anc) * (kTileN * 4 + 4 + M * 4);
 }
 
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
@@ -73,6 +90,17 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
     // the other two counters are left at "do not wait"
     static_assert(N >= 0 && N < 64, "vmcnt has 6 bits");
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// Waits until at most `tiles` tiles' worth of this wave's global->LDS transfers
+// (kPerTile instructions each, retired in order) are still outstanding.
+template <int kPerTile> __device__ __forceinline__ void wait_tiles_outstanding(int tiles) {
+    static_assert((kMaxStages - 2) * kPerTile < 64, "ring too deep for vmcnt");
+    switch (tiles) {
+        case 0: wait_vmcnt<0>(); break;
+        case 1: wait_vmcnt<kPerTile>(); break;
+        default: wait_vmcnt<2 * kPerTile>(); break;
+    }
 }
 
 // 32-bit LDS address of a pointer into the dynamic shared segment
@@ -115,8 +143,6 @@ template <> __device__ __forceinline__ void wait_lds<4>(VPair (&f)[2][4]) {
                    "+v"(f[1][2].a), "+v"(f[1][2].b), "+v"(f[1][3].a), "+v"(f[1][3].b) :: "memory");
 }
 
-constexpr int stages_for(int block_m) { return block_m == 128 ? 4 : 3; }
-
 // 16-byte chunk position of (row, chunk) inside an LDS tile.  K is read as whole
 // 16-byte fragments by 32 different rows at once, V as 4-row x 64-byte groups by
 // the transposing read; each gets the XOR pattern that spreads its access over
@@ -131,12 +157,11 @@ template <int D> __device__ __forceinline__ int v_chunk(int row, int c) {
 }
 
 template <bool BF16, int D, int M, bool SPLIT>
-__global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p) {
+__global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int stages) {
     using MM = Mma<BF16>;
     using T = typename MM::elem;
+    using T2 = typename MM::elem2;
     using Frag = typename MM::frag;
-    constexpr int kStages = stages_for(M);
-    constexpr int kAhead = kStages - 1;           // tiles in flight beyond the one being used
     constexpr int kWaves = M / 32;
     constexpr int kThreads = kWaves * 64;
     constexpr int kCpr = D / 8;                   // 16-byte chunks per row
@@ -144,14 +169,15 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p) {
     constexpr int kDmaPerTile = 2 * kTileN / kRowsPerDma;   // K and V transfers of one tile
     constexpr int kDmaPerWave = kDmaPerTile / kWaves;
     static_assert(kDmaPerWave * kWaves == kDmaPerTile, "transfers must split evenly over the waves");
+    constexpr int kRowGroups = (kDmaPerWave + 1) / 2;   // row groups a wave touches per tile
     constexpr int kSteps = D / 16;                // QK^T MFMAs per tile
     constexpr int kDTiles = D / 32;               // 32-row tiles of O^T
     constexpr int kTileElems = kTileN * D;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    T* ring = reinterpret_cast<T*>(smem);                 // [kStages][K tile | V tile]
-    int* key_s = reinterpret_cast<int*>(ring + kStages * 2 * kTileElems);
-    const int cap = anc_tile_capacity(p.max_anc);
+    T* ring = reinterpret_cast<T*>(smem);                 // [stages][K tile | V tile]
+    int* key_s = reinterpret_cast<int*>(ring + stages * 2 * kTileElems);
+    const int cap = anc_tile_capacity(p.max_anc);                            // listed tiles
     uint32_t* valid_s = reinterpret_cast<uint32_t*>(key_s + cap * kTileN);   // [cap]
     uint32_t* mask_s = valid_s + cap;                                        // [cap][M]
 
@@ -177,15 +203,69 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p) {
     const T* kb = static_cast<const T*>(p.k) + (size_t)hz * p.nk * D;
     const T* vb = static_cast<const T*>(p.v) + (size_t)hz * p.nk * D;
 
+    // ---- block metadata: the loads nothing else depends on go out first --------
     int n_anc = p.anc_count ? p.anc_count[j] : p.max_anc;
-    n_anc = min(max(n_anc, 0), p.max_anc);
-    const int anc_tiles = (n_anc + kTileN - 1) / kTileN;
-    const int prefix_tiles = (p.prefix + kTileN - 1) / kTileN;
-    const int total_tiles = anc_tiles + prefix_tiles;
-
-    // ---- everything that does not depend on other loads goes out first ---------
     const int64_t leaf64 = p.leaf_idx[(size_t)j * M + row_in_block];
-    // Q fragments: B operand of S^T = K.Q^T, lane holds Q[q][16s + 8h .. +7]
+    // Sanitised ancestor list.  An empty or out-of-range slot is given the row of the
+    // first valid key of its tile (row 0 if the tile has none): the transfer count per
+    // tile stays fixed, the slot's mask bits are cleared through valid_s, and the data
+    // it brings in is data the tile holds anyway.
+    for (int c = tid; c < cap * kTileN; c += kThreads) {
+        int64_t idx = -1;
+        if (c < p.max_anc) idx = p.ancestor_idx[(size_t)j * p.max_anc + c];
+        const bool ok = idx >= 0 && idx < p.nk;
+        const uint64_t vote = __ballot(ok);
+        const uint32_t mine = (uint32_t)(vote >> (lane & 32));
+        const int first = mine ? (lane & 32) + __ffs(mine) - 1 : lane;
+        const int fallback = __shfl(ok ? (int)idx : 0, first);
+        key_s[c] = ok ? (int)idx : fallback;
+        if ((lane & 31) == 0) valid_s[c >> 5] = mine;
+    }
+    {
+        const uint32_t* src = p.mask_bits + (size_t)j * p.mask_words * M;
+        for (int e = tid; e < p.mask_words * M; e += kThreads) mask_s[e] = src[e];
+    }
+    n_anc = min(max(n_anc, 0), p.max_anc);
+    const int listed_tiles = (n_anc + kTileN - 1) / kTileN;
+    const int total_tiles = listed_tiles + (p.prefix + kTileN - 1) / kTileN;
+    const int ahead = stages - 1;   // tiles kept in flight beyond the one in use
+    __syncthreads();
+
+    // ---- gather: HBM -> LDS, 16 bytes per lane, no registers in between --------
+    // Transfer g of a tile moves row group g/2 = rows [kRowsPerDma*(g/2), +kRowsPerDma) of K
+    // (g even) or V (g odd); wave w issues transfers [w*kDmaPerWave, +kDmaPerWave).  Lane i
+    // lands at LDS byte 16*i of the transfer, i.e. row i / kCpr, chunk slot i % kCpr, and
+    // fetches the chunk that the XOR swizzle assigns to that slot.  Every wave issues exactly
+    // kDmaPerWave transfers per tile: the vmcnt bookkeeping below counts on it.
+    const int dma_row = lane / kCpr, dma_slot = lane % kCpr;
+    auto issue = [&](int t, int stage) {
+        T* dst_tile = ring + stage * 2 * kTileElems;
+        int rows[kRowGroups];
+#pragma unroll
+        for (int i = 0; i < kRowGroups; ++i) {
+            const int r = ((wave * kDmaPerWave) / 2 + i) * kRowsPerDma + dma_row;
+            if (t < listed_tiles) rows[i] = key_s[t * kTileN + r];
+            else rows[i] = min((t - listed_tiles) * kTileN + r, p.prefix - 1);
+        }
+#pragma unroll
+        for (int i = 0; i < kDmaPerWave; ++i) {
+            const int g = wave * kDmaPerWave + i;
+            const int u = g >> 1;
+            const bool is_v = g & 1;
+            const int r = u * kRowsPerDma + dma_row;
+            const size_t row_off = (size_t)rows[u - (wave * kDmaPerWave) / 2] * D;
+            const T* src = is_v ? vb + row_off + v_chunk<D>(r, dma_slot) * 8
+                                : kb + row_off + k_chunk<D>(r, dma_slot) * 8;
+            __builtin_amdgcn_global_load_lds(
+                (const void __attribute__((address_space(1)))*)src,
+                (void __attribute__((address_space(3)))*)(dst_tile + (is_v ? kTileElems : 0) + u * 512),
+                16, 0, 0);
+        }
+    };
+    for (int t = 0; t < ahead; ++t)
+        if (t < total_tiles) issue(t, t);
+
+    // ---- Q fragments: B operand of S^T = K.Q^T, lane holds Q[q][16s + 8h .. +7] --
     Frag qf[kSteps];
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
@@ -193,56 +273,10 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p) {
         if (q_ok) raw = *reinterpret_cast<const u32x4*>(qb + (size_t)qrow * D + 16 * s + 8 * h);
         qf[s] = __builtin_bit_cast(Frag, raw);
     }
-    // sanitised ancestor list, per-tile validity words, this block's mask words
-    for (int c = tid; c < anc_tiles * kTileN; c += kThreads) {
-        int64_t idx = -1;
-        if (c < n_anc) idx = p.ancestor_idx[(size_t)j * p.max_anc + c];
-        const bool ok = idx >= 0 && idx < p.nk;
-        key_s[c] = ok ? (int)idx : -1;
-        const uint64_t vote = __ballot(ok);
-        if (lane == 0) valid_s[c >> 5] = (uint32_t)vote;
-        if (lane == 32) valid_s[c >> 5] = (uint32_t)(vote >> 32);
-    }
-    {
-        const uint32_t* src = p.mask_bits + (size_t)j * p.mask_words * M;
-        for (int e = tid; e < anc_tiles * M; e += kThreads) mask_s[e] = src[e];
-    }
-    // Rows of a partly filled tile are not transferred; whatever a V buffer holds
-    // there meets a weight of exactly 0, so it only has to be finite: start from zeros.
-    for (int e = tid; e < kStages * kTileElems / 8; e += kThreads) {
-        const int stage = e / (kTileElems / 8), off = e % (kTileElems / 8);
-        *reinterpret_cast<u32x4*>(ring + (stage * 2 + 1) * kTileElems + off * 8) = u32x4{0u, 0u, 0u, 0u};
-    }
-    __syncthreads();
-
-    // ---- gather: HBM -> LDS, 16 bytes per lane, no registers in between --------
-    // Transfer g of a tile moves rows [kRowsPerDma*u, +kRowsPerDma) of K (g < half) or V.
-    // Lane i lands at LDS byte 16*i of the transfer, i.e. row i / kCpr, chunk slot i % kCpr;
-    // it fetches the chunk that the XOR swizzle assigns to that slot.
-    auto issue = [&](int t) {
-        T* stage = ring + (t % kStages) * 2 * kTileElems;
-#pragma unroll
-        for (int i = 0; i < kDmaPerWave; ++i) {
-            const int g = wave * kDmaPerWave + i;
-            const bool is_v = g >= kDmaPerTile / 2;
-            const int u = is_v ? g - kDmaPerTile / 2 : g;
-            const int r = u * kRowsPerDma + lane / kCpr;
-            const int slot = lane % kCpr;
-            int row;
-            if (t < anc_tiles) row = key_s[t * kTileN + r];
-            else { row = (t - anc_tiles) * kTileN + r; if (row >= p.prefix) row = -1; }
-            const int c = is_v ? v_chunk<D>(r, slot) : k_chunk<D>(r, slot);
-            const T* src = (is_v ? vb : kb) + (size_t)max(row, 0) * D + c * 8;
-            T* dst = stage + (is_v ? kTileElems : 0) + u * 512;
-            if (row >= 0)
-                __builtin_amdgcn_global_load_lds(
-                    (const void __attribute__((address_space(1)))*)src,
-                    (void __attribute__((address_space(3)))*)dst, 16, 0, 0);
-        }
-    };
 
     // ---- leaf (diagonal) path seeds the running softmax -----------------------
-    // reference fstattention.py:86-91,104-107: row r also attends to K/V row leaf_idx[j, r]
+    // reference fstattention.py:86-91,104-107: row r also attends to K/V row leaf_idx[j, r].
+    // One key per query: every lane dots its Q registers with its own row, no LDS.
     float m_i = -INFINITY, l_i = 0.f;
     f32x16 o[kDTiles];
     {
@@ -263,17 +297,16 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p) {
                 vraw[dt][g] = u32x2{0u, 0u};
                 if (leaf_ok) vraw[dt][g] = *reinterpret_cast<const u32x2*>(vb + leaf * D + 32 * dt + 8 * g + 4 * h);
             }
-        // the first tiles start moving before the leaf rows are used
-#pragma unroll
-        for (int t = 0; t < kAhead; ++t)
-            if (t < total_tiles) issue(t);
-
         float part = 0.f;
 #pragma unroll
         for (int s = 0; s < kSteps; ++s) {
-            const Frag kf = __builtin_bit_cast(Frag, kraw[s]);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) part += MM::to_f32(qf[s][e]) * MM::to_f32(kf[e]);
+            for (int e = 0; e < 4; ++e) {
+                const T2 a = {qf[s][2 * e], qf[s][2 * e + 1]};
+                const Frag kf = __builtin_bit_cast(Frag, kraw[s]);
+                const T2 b = {kf[2 * e], kf[2 * e + 1]};
+                part = MM::dot2(a, b, part);
+            }
         }
         const float dot = part + __shfl_xor(part, 32);
         if (leaf_ok) { m_i = dot * p.scale_log2e; l_i = h == 0 ? 1.f : 0.f; }
@@ -284,24 +317,27 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p) {
                 typedef T t4 __attribute__((ext_vector_type(4)));
                 const t4 vv = __builtin_bit_cast(t4, vraw[dt][g]);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) o[dt][4 * g + e] = MM::to_f32(vv[e]);
+                for (int e = 0; e < 4; ++e) o[dt][4 * g + e] = (float)vv[e];
             }
     }
 
+    int stage = 0;                      // ring slot of tile t
+    int fill = ahead % stages;          // ring slot the next issued tile goes to (= slot of tile t-1)
     for (int t = 0; t < total_tiles; ++t) {
-        // tile t has landed once at most the transfers of the tiles behind it are outstanding
-        if (total_tiles - 1 - t >= kAhead - 1) wait_vmcnt<(kAhead - 1) * kDmaPerWave>();
-        else wait_vmcnt<0>();
+        // tile t has landed once at most the transfers of the tiles issued after it are outstanding
+        wait_tiles_outstanding<kDmaPerWave>(min(total_tiles - 1 - t, ahead - 1));
         __syncthreads();   // everyone's share of tile t is in LDS; everyone is done with tile t-1
-        if (t + kAhead < total_tiles) issue(t + kAhead);   // reuses the buffer of tile t-1
-
-        const T* kt = ring + (t % kStages) * 2 * kTileElems;
+        if (t + ahead < total_tiles) issue(t + ahead, fill);
+        const T* kt = ring + stage * 2 * kTileElems;
         const T* vt = kt + kTileElems;
+        fill = stage;
+        stage = stage + 1 == stages ? 0 : stage + 1;
+
         uint32_t word;
-        if (t < anc_tiles) {
+        if (t < listed_tiles) {
             word = mask_s[t * M + row_in_block] & valid_s[t];
         } else {
-            const int left = p.prefix - (t - anc_tiles) * kTileN;
+            const int left = p.prefix - (t - listed_tiles) * kTileN;
             word = left >= 32 ? 0xffffffffu : ((1u << left) - 1u);
         }
         if (__ballot(word != 0u) == 0ull) continue;   // none of this wave's queries attends to the tile
@@ -344,37 +380,47 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p) {
             mx = fmaxf(mx, sv[r]);
         }
         mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_i, mx);
-        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_i - m_safe);
+        // Raise the running maximum only for rows that would otherwise produce a weight
+        // above 2^kRescaleSlack (always when the row had no key so far); rare after the
+        // first tiles, so the rescale of the accumulators is a wave-uniform branch.
+        const bool raise = mx > m_i + kRescaleSlack || (m_i == -INFINITY && mx > -INFINITY);
+        if (__ballot(raise) != 0ull) {
+            const float alpha = raise ? __builtin_amdgcn_exp2f(m_i - mx) : 1.f;   // exp2(-inf) = 0
+            if (raise) m_i = mx;
+            l_i *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < kDTiles; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+        }
+        const float m_safe = m_i == -INFINITY ? 0.f : m_i;
         float rowsum = 0.f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             sv[r] = __builtin_amdgcn_exp2f(sv[r] - m_safe);
             rowsum += sv[r];
         }
-        l_i = l_i * alpha + rowsum;
-        m_i = m_new;
-        if (__ballot(alpha != 1.f) != 0ull) {
-#pragma unroll
-            for (int dt = 0; dt < kDTiles; ++dt)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
-        }
+        l_i += rowsum;
         // P^T fragments: registers 8kk .. 8kk+7 are the 8 k-indices this lane feeds to MFMA kk
         Frag ph[2], pl[2];
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float w = sv[8 * kk + e];
-                const T hi = (T)w;
-                ph[kk][e] = hi;
-                if (SPLIT) pl[kk][e] = (T)(w - MM::to_f32(hi));
+            for (int e = 0; e < 8; e += 2) {
+                const f32x2 w = {sv[8 * kk + e], sv[8 * kk + e + 1]};
+                const T2 hi = __builtin_convertvector(w, T2);
+                ph[kk][e] = hi[0];
+                ph[kk][e + 1] = hi[1];
+                if (SPLIT) {
+                    const f32x2 rest = w - __builtin_convertvector(hi, f32x2);
+                    const T2 lo = __builtin_convertvector(rest, T2);
+                    pl[kk][e] = lo[0];
+                    pl[kk][e + 1] = lo[1];
+                }
             }
         }
         // O^T += V_tile^T . P^T ; hi weights of all head-dim tiles first, then lo, so that
-        // MFMAs on the same accumulator are four instructions apart
+        // MFMAs on the same accumulator are several instructions apart
         wait_lds(vfrag);
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
@@ -400,6 +446,7 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p) {
         for (int dt = 0; dt < kDTiles; ++dt) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
+                // accumulator rows 8g + 4h .. +3 of tile dt are 4 consecutive head dims
                 const int d = 32 * dt + 8 * g + 4 * h;
                 float4 val;
                 val.x = o[dt][4 * g + 0] * inv;
@@ -410,8 +457,10 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p) {
                     *reinterpret_cast<float4*>(static_cast<float*>(p.o) + base + d) = val;
                 } else {
                     typedef T t4 __attribute__((ext_vector_type(4)));
+                    const T2 lo = __builtin_convertvector((f32x2){val.x, val.y}, T2);
+                    const T2 hi = __builtin_convertvector((f32x2){val.z, val.w}, T2);
                     t4 packed;
-                    packed[0] = (T)val.x; packed[1] = (T)val.y; packed[2] = (T)val.z; packed[3] = (T)val.w;
+                    packed[0] = lo[0]; packed[1] = lo[1]; packed[2] = hi[0]; packed[3] = hi[1];
                     *reinterpret_cast<t4*>(static_cast<T*>(p.o) + base + d) = packed;
                 }
             }
@@ -421,7 +470,11 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p) {
 
 template <bool BF16, int D, int M, bool SPLIT>
 int launch_one(const AttnParams& p, hipStream_t stream) {
-    const size_t lds = mfma_lds_bytes<D, M, stages_for(M)>(p.max_anc);
+    // ring depth: everything in flight at once for short tile lists, else the limit
+    const int tiles = anc_tile_capacity(p.max_anc) + (p.prefix + kTileN - 1) / kTileN;
+    int stages = tiles < 2 ? 2 : (tiles > kMaxStages ? kMaxStages : tiles);
+    size_t lds = mfma_lds_bytes<D, M>(p.max_anc, stages);
+    while (lds > 160 * 1024 && stages > 2) lds = mfma_lds_bytes<D, M>(p.max_anc, --stages);
     if (lds > 160 * 1024)
         return fail(FSTA_EUNSUPPORTED, "max_ancestors=%d needs %zu bytes of LDS (limit 163840)", p.max_anc, lds);
     if (lds > 64 * 1024)
@@ -429,7 +482,7 @@ int launch_one(const AttnParams& p, hipStream_t stream) {
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
     const unsigned grid = (unsigned)(kXcds * slices_per_xcd * p.nb);
-    hipLaunchKernelGGL((attn_mfma_kernel<BF16, D, M, SPLIT>), dim3(grid), dim3(M * 2), lds, stream, p);
+    hipLaunchKernelGGL((attn_mfma_kernel<BF16, D, M, SPLIT>), dim3(grid), dim3(M * 2), lds, stream, p, stages);
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
 }

@@ -155,7 +155,9 @@ def test_fast_pv_flag_stays_within_loose_bound():
     want, _ = dense_oracle(q, k, v, cfg.parent, scale)
     o = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(), scale,
                       BLOCK_M=cfg.block_m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32, fast_pv=True)
-    assert (o.cpu().double() - want).abs().max() < 1e-2
+    # one bf16 rounding per weight: |err| <= 2^-9 * max|v|, and max|v| of N(0,1) samples is ~5
+    err = float((o.cpu().double() - want).abs().max())
+    assert err < 2.0 ** -9 * float(v.abs().max()), err
 
 
 def test_ancestor_slots_with_holes_and_out_of_range_ids_are_skipped():
