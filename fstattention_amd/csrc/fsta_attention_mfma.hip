@@ -3,12 +3,15 @@
 //
 // One workgroup owns one query block of one (batch, head) slice; each of its
 // M/32 waves owns 32 query rows and keeps their state in registers for the whole
-// kernel.  The block's own rows (the "leaf" diagonal of reference
-// fstattention.py:86-91,104-107: one key per query) never go through LDS: every
-// lane dots its Q registers with its own leaf row and seeds the running softmax
-// with it.  All other keys are processed in tiles of 32: first the block's unique
-// ancestors under the packed tree mask, then the dense shared prefix
-// (fstattention.py:113-136).  Work per tile:
+// kernel.  Keys come in tiles of 32 rows, gathered through LDS.  The tile list is
+//
+//   [ M/32 leaf tiles | ancestor tiles | shared-prefix tiles ]
+//
+// Leaf tile w holds K/V rows leaf_idx[j, 32w .. 32w+31] (the diagonal of reference
+// fstattention.py:86-91,104-107: one key per query); wave w takes one dot product
+// per query from it on the vector ALU and seeds its running softmax.  Ancestor
+// tiles carry the packed tree mask, prefix tiles are dense
+// (fstattention.py:113-136); work per such tile:
 //
 //   S^T[key, q] = K_tile . Q^T        v_mfma_f32_32x32x16, K fragments from LDS,
 //                                     Q fragments loaded once from HBM into VGPRs
@@ -62,6 +65,15 @@ template <> struct Mma<true> {
     static __device__ __forceinline__ float dot2(elem2 a, elem2 b, float c) {
         return __builtin_amdgcn_fdot2_f32_bf16(a, b, c, false);
     }
+    // Two floats -> two bf16 (round to nearest even) in one dword, first value in the low
+    // half: one v_cvt_pk_bf16_f32.  Kept as a vector cast the compiler can see (not inline
+    // assembly), so that it inserts the wait states the matrix cores need after a VALU write.
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        const f32x2 w = {a, b};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(w, bf16x2));
+    }
+    static __device__ __forceinline__ float low(uint32_t pk) { return __builtin_bit_cast(float, pk << 16); }
+    static __device__ __forceinline__ float high(uint32_t pk) { return __builtin_bit_cast(float, pk & 0xffff0000u); }
 };
 template <> struct Mma<false> {
     using elem = _Float16;
@@ -73,16 +85,29 @@ template <> struct Mma<false> {
     static __device__ __forceinline__ float dot2(elem2 a, elem2 b, float c) {
         return __builtin_amdgcn_fdot2(a, b, c, false);
     }
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        const uint32_t lo = __builtin_bit_cast(unsigned short, (_Float16)a);
+        const uint32_t hi = __builtin_bit_cast(unsigned short, (_Float16)b);
+        return lo | (hi << 16);
+    }
+    static __device__ __forceinline__ float low(uint32_t pk) {
+        return (float)__builtin_bit_cast(_Float16, (unsigned short)(pk & 0xffffu));
+    }
+    static __device__ __forceinline__ float high(uint32_t pk) {
+        return (float)__builtin_bit_cast(_Float16, (unsigned short)(pk >> 16));
+    }
 };
 
 __host__ __device__ constexpr int anc_tile_capacity(int max_anc) { return (max_anc + kTileN - 1) / kTileN; }
 
-// LDS of one workgroup: ring of K|V tiles, then per ancestor tile 32 sanitised keys,
-// one validity word and M mask words.
+// LDS of one workgroup: ring of K|V tiles, then 32 sanitised keys and a validity word
+// per listed tile (M/32 leaf tiles, then the ancestor tiles) and M mask words per
+// ancestor tile.
 template <int D, int M>
 __host__ __device__ constexpr size_t mfma_lds_bytes(int max_anc, int stages) {
     return (size_t)stages * 2 * kTileN * D * 2 +
-           (size_t)anc_tile_capacity(max_anc) * (kTileN * 4 + 4 + M * 4);
+           (size_t)(M / 32 + anc_tile_capacity(max_anc)) * (kTileN * 4 + 4) +
+           (size_t)anc_tile_capacity(max_anc) * M * 4;
 }
 
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
@@ -108,40 +133,36 @@ __device__ __forceinline__ uint32_t lds_addr(const void* ptr) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)ptr;
 }
 
+// LDS reads of tile data are issued as inline assembly on purpose: for the builtin
+// forms the compiler's wait-count pass first drains every outstanding global->LDS
+// transfer (s_waitcnt vmcnt(0)), which would empty the gather ring on every tile.
+// A result is only valid after lds_wait() followed by lds_tie() on it.
+//
 // ds_read_b64_tr_b16: within each group of 16 lanes, lane i supplies the address of
 // 4 consecutive 16-bit elements (think row i/4, column block i%4 of a 4 x 16 tile)
 // and receives element column i of rows 0..3, i.e. component j comes from lane
-// 4j + i/4, element i%4.  It is issued as inline assembly on purpose: the compiler
-// orders the builtin form behind every outstanding global->LDS transfer
-// (s_waitcnt vmcnt(0)), which would drain the gather ring on every tile.  The
-// result is only valid after wait_lds() has been applied to it.
+// 4j + i/4, element i%4.
 __device__ __forceinline__ s16x4 lds_read_tr16(uint32_t addr) {
     s16x4 out;
     asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(out) : "v"(addr) : "memory");
     return out;
 }
+__device__ __forceinline__ u32x4 lds_read_b128(uint32_t addr) {
+    u32x4 out;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(out) : "v"(addr) : "memory");
+    return out;
+}
+__device__ __forceinline__ u32x2 lds_read_b64(uint32_t addr) {
+    u32x2 out;
+    asm volatile("ds_read_b64 %0, %1" : "=v"(out) : "v"(addr) : "memory");
+    return out;
+}
+// Waits for every outstanding LDS access of this wave.
+__device__ __forceinline__ void lds_wait() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+// Orders every later use of `x` behind the preceding lds_wait().
+template <typename V> __device__ __forceinline__ void lds_tie(V& x) { asm volatile("" : "+v"(x)); }
 
 struct VPair { s16x4 a, b; };   // 8 consecutive k-indices of one A-operand row
-
-// Waits for every outstanding LDS access and ties the fragments to the wait, so no
-// use of them can be scheduled ahead of it.
-template <int N> __device__ __forceinline__ void wait_lds(VPair (&f)[2][N]);
-template <> __device__ __forceinline__ void wait_lds<1>(VPair (&f)[2][1]) {
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(f[0][0].a), "+v"(f[0][0].b), "+v"(f[1][0].a), "+v"(f[1][0].b) :: "memory");
-}
-template <> __device__ __forceinline__ void wait_lds<2>(VPair (&f)[2][2]) {
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(f[0][0].a), "+v"(f[0][0].b), "+v"(f[0][1].a), "+v"(f[0][1].b),
-                   "+v"(f[1][0].a), "+v"(f[1][0].b), "+v"(f[1][1].a), "+v"(f[1][1].b) :: "memory");
-}
-template <> __device__ __forceinline__ void wait_lds<4>(VPair (&f)[2][4]) {
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(f[0][0].a), "+v"(f[0][0].b), "+v"(f[0][1].a), "+v"(f[0][1].b),
-                   "+v"(f[0][2].a), "+v"(f[0][2].b), "+v"(f[0][3].a), "+v"(f[0][3].b),
-                   "+v"(f[1][0].a), "+v"(f[1][0].b), "+v"(f[1][1].a), "+v"(f[1][1].b),
-                   "+v"(f[1][2].a), "+v"(f[1][2].b), "+v"(f[1][3].a), "+v"(f[1][3].b) :: "memory");
-}
 
 // 16-byte chunk position of (row, chunk) inside an LDS tile.  K is read as whole
 // 16-byte fragments by 32 different rows at once, V as 4-row x 64-byte groups by
@@ -177,9 +198,9 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     T* ring = reinterpret_cast<T*>(smem);                 // [stages][K tile | V tile]
     int* key_s = reinterpret_cast<int*>(ring + stages * 2 * kTileElems);
-    const int cap = anc_tile_capacity(p.max_anc);                            // listed tiles
+    const int cap = kWaves + anc_tile_capacity(p.max_anc);                   // listed tiles
     uint32_t* valid_s = reinterpret_cast<uint32_t*>(key_s + cap * kTileN);   // [cap]
-    uint32_t* mask_s = valid_s + cap;                                        // [cap][M]
+    uint32_t* mask_s = valid_s + cap;                                        // [ancestor tiles][M]
 
     // Workgroup -> (slice, block): consecutive workgroup ids rotate over the 8
     // XCDs, so give every XCD whole (batch, head) slices; all query blocks of a
@@ -206,13 +227,16 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
     // ---- block metadata: the loads nothing else depends on go out first --------
     int n_anc = p.anc_count ? p.anc_count[j] : p.max_anc;
     const int64_t leaf64 = p.leaf_idx[(size_t)j * M + row_in_block];
-    // Sanitised ancestor list.  An empty or out-of-range slot is given the row of the
-    // first valid key of its tile (row 0 if the tile has none): the transfer count per
-    // tile stays fixed, the slot's mask bits are cleared through valid_s, and the data
-    // it brings in is data the tile holds anyway.
+    const bool leaf_ok = leaf64 >= 0 && leaf64 < p.nk;
+    // Sanitised key lists: the block's M leaf slots (tiles 0 .. kWaves-1), then the
+    // ancestor slots.  An empty or out-of-range slot is given the row of the first valid
+    // key of its tile (row 0 if the tile has none): the transfer count per tile stays
+    // fixed, the slot's mask bits are cleared through valid_s, and the data it brings in
+    // is data the tile holds anyway.
     for (int c = tid; c < cap * kTileN; c += kThreads) {
         int64_t idx = -1;
-        if (c < p.max_anc) idx = p.ancestor_idx[(size_t)j * p.max_anc + c];
+        if (c < M) idx = p.leaf_idx[(size_t)j * M + c];
+        else if (c - M < p.max_anc) idx = p.ancestor_idx[(size_t)j * p.max_anc + (c - M)];
         const bool ok = idx >= 0 && idx < p.nk;
         const uint64_t vote = __ballot(ok);
         const uint32_t mine = (uint32_t)(vote >> (lane & 32));
@@ -225,8 +249,17 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
         const uint32_t* src = p.mask_bits + (size_t)j * p.mask_words * M;
         for (int e = tid; e < p.mask_words * M; e += kThreads) mask_s[e] = src[e];
     }
+    // Q fragments: B operand of S^T = K.Q^T, lane holds Q[q][16s + 8h .. +7].  Requested
+    // after the lists so that waiting for the lists does not wait for Q.
+    Frag qf[kSteps];
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) {
+        u32x4 raw = {0u, 0u, 0u, 0u};
+        if (q_ok) raw = *reinterpret_cast<const u32x4*>(qb + (size_t)qrow * D + 16 * s + 8 * h);
+        qf[s] = __builtin_bit_cast(Frag, raw);
+    }
     n_anc = min(max(n_anc, 0), p.max_anc);
-    const int listed_tiles = (n_anc + kTileN - 1) / kTileN;
+    const int listed_tiles = kWaves + (n_anc + kTileN - 1) / kTileN;
     const int total_tiles = listed_tiles + (p.prefix + kTileN - 1) / kTileN;
     const int ahead = stages - 1;   // tiles kept in flight beyond the one in use
     __syncthreads();
@@ -254,7 +287,8 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
             const bool is_v = g & 1;
             const int r = u * kRowsPerDma + dma_row;
             const size_t row_off = (size_t)rows[u - (wave * kDmaPerWave) / 2] * D;
-            const T* src = is_v ? vb + row_off + v_chunk<D>(r, dma_slot) * 8
+            // V of a leaf tile is read row-wise like K (no transposing read), so it takes K's swizzle
+            const T* src = is_v ? vb + row_off + (t < kWaves ? k_chunk<D>(r, dma_slot) : v_chunk<D>(r, dma_slot)) * 8
                                 : kb + row_off + k_chunk<D>(r, dma_slot) * 8;
             __builtin_amdgcn_global_load_lds(
                 (const void __attribute__((address_space(1)))*)src,
@@ -265,83 +299,89 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
     for (int t = 0; t < ahead; ++t)
         if (t < total_tiles) issue(t, t);
 
-    // ---- Q fragments: B operand of S^T = K.Q^T, lane holds Q[q][16s + 8h .. +7] --
-    Frag qf[kSteps];
-#pragma unroll
-    for (int s = 0; s < kSteps; ++s) {
-        u32x4 raw = {0u, 0u, 0u, 0u};
-        if (q_ok) raw = *reinterpret_cast<const u32x4*>(qb + (size_t)qrow * D + 16 * s + 8 * h);
-        qf[s] = __builtin_bit_cast(Frag, raw);
-    }
-
-    // ---- leaf (diagonal) path seeds the running softmax -----------------------
-    // reference fstattention.py:86-91,104-107: row r also attends to K/V row leaf_idx[j, r].
-    // One key per query: every lane dots its Q registers with its own row, no LDS.
     float m_i = -INFINITY, l_i = 0.f;
     f32x16 o[kDTiles];
-    {
-        const bool leaf_ok = leaf64 >= 0 && leaf64 < p.nk;
-        const size_t leaf = leaf_ok ? (size_t)leaf64 : 0;
-        u32x4 kraw[kSteps];
-        u32x2 vraw[kDTiles][4];
 #pragma unroll
-        for (int s = 0; s < kSteps; ++s) {
-            kraw[s] = u32x4{0u, 0u, 0u, 0u};
-            if (leaf_ok) kraw[s] = *reinterpret_cast<const u32x4*>(kb + leaf * D + 16 * s + 8 * h);
-        }
+    for (int dt = 0; dt < kDTiles; ++dt)
 #pragma unroll
-        for (int dt = 0; dt < kDTiles; ++dt)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                // accumulator rows 8g + 4h .. +3 of tile dt are 4 consecutive head dims
-                vraw[dt][g] = u32x2{0u, 0u};
-                if (leaf_ok) vraw[dt][g] = *reinterpret_cast<const u32x2*>(vb + leaf * D + 32 * dt + 8 * g + 4 * h);
-            }
-        float part = 0.f;
-#pragma unroll
-        for (int s = 0; s < kSteps; ++s) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const T2 a = {qf[s][2 * e], qf[s][2 * e + 1]};
-                const Frag kf = __builtin_bit_cast(Frag, kraw[s]);
-                const T2 b = {kf[2 * e], kf[2 * e + 1]};
-                part = MM::dot2(a, b, part);
-            }
-        }
-        const float dot = part + __shfl_xor(part, 32);
-        if (leaf_ok) { m_i = dot * p.scale_log2e; l_i = h == 0 ? 1.f : 0.f; }
-#pragma unroll
-        for (int dt = 0; dt < kDTiles; ++dt)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                typedef T t4 __attribute__((ext_vector_type(4)));
-                const t4 vv = __builtin_bit_cast(t4, vraw[dt][g]);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) o[dt][4 * g + e] = (float)vv[e];
-            }
-    }
+        for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
 
     int stage = 0;                      // ring slot of tile t
     int fill = ahead % stages;          // ring slot the next issued tile goes to (= slot of tile t-1)
-    for (int t = 0; t < total_tiles; ++t) {
-        // tile t has landed once at most the transfers of the tiles issued after it are outstanding
+    const T* kt;                        // K tile of the current step; V follows it
+    // Start of step t: tile t has landed once at most the transfers of the tiles issued
+    // after it are outstanding; after the barrier everyone's share of it is in LDS and
+    // everyone is done with tile t-1, whose slot takes the next gather.
+    auto begin_step = [&](int t) {
         wait_tiles_outstanding<kDmaPerWave>(min(total_tiles - 1 - t, ahead - 1));
-        __syncthreads();   // everyone's share of tile t is in LDS; everyone is done with tile t-1
+        __syncthreads();
         if (t + ahead < total_tiles) issue(t + ahead, fill);
-        const T* kt = ring + stage * 2 * kTileElems;
-        const T* vt = kt + kTileElems;
+        kt = ring + stage * 2 * kTileElems;
         fill = stage;
         stage = stage + 1 == stages ? 0 : stage + 1;
+    };
 
+    // Leaf tile t = the block's own rows 32t .. 32t+31 (reference
+    // fstattention.py:86-91,104-107): query r sees exactly row r of it, so this is one
+    // dot product per lane pair for wave t, no matrix core; it seeds the running softmax.
+    for (int t = 0; t < kWaves; ++t) {
+        begin_step(t);
+        const T* vt = kt + kTileElems;
+        if (t == wave && __ballot(leaf_ok) != 0ull) {
+            float part = 0.f;
+            {
+                u32x4 kraw[kSteps];
+#pragma unroll
+                for (int ks = 0; ks < kSteps; ++ks)
+                    kraw[ks] = lds_read_b128(lds_addr(kt + ql * D + k_chunk<D>(ql, 2 * ks + h) * 8));
+                lds_wait();
+#pragma unroll
+                for (int ks = 0; ks < kSteps; ++ks) {
+                    lds_tie(kraw[ks]);
+                    const Frag kf = __builtin_bit_cast(Frag, kraw[ks]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const T2 a = {qf[ks][2 * e], qf[ks][2 * e + 1]};
+                        const T2 b = {kf[2 * e], kf[2 * e + 1]};
+                        part = MM::dot2(a, b, part);
+                    }
+                }
+            }
+            const float dot = part + __shfl_xor(part, 32);
+            if (leaf_ok) { m_i = dot * p.scale_log2e; l_i = h == 0 ? 1.f : 0.f; }
+#pragma unroll
+            for (int dt = 0; dt < kDTiles; ++dt) {
+                u32x2 vraw[4];
+#pragma unroll
+                for (int g = 0; g < 4; ++g)   // accumulator rows 8g + 4h .. +3 of tile dt: 4 head dims
+                    vraw[g] = lds_read_b64(lds_addr(vt + ql * D + k_chunk<D>(ql, 4 * dt + g) * 8 + 4 * h));
+                lds_wait();
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    lds_tie(vraw[g]);
+                    const uint32_t w0 = vraw[g][0], w1 = vraw[g][1];
+                    o[dt][4 * g + 0] = leaf_ok ? MM::low(w0) : 0.f;
+                    o[dt][4 * g + 1] = leaf_ok ? MM::high(w0) : 0.f;
+                    o[dt][4 * g + 2] = leaf_ok ? MM::low(w1) : 0.f;
+                    o[dt][4 * g + 3] = leaf_ok ? MM::high(w1) : 0.f;
+                }
+            }
+        }
+    }
+
+    // Ancestor tiles under the packed tree mask, then the dense shared prefix.  A tile none
+    // of this wave's queries attends to is not skipped: with an all-zero mask word it adds
+    // exact zeros, and a branch-free body spares the accumulators a copy per step.
+    for (int t = kWaves; t < total_tiles; ++t) {
+        begin_step(t);
+        const T* vt = kt + kTileElems;
         uint32_t word;
         if (t < listed_tiles) {
-            word = mask_s[t * M + row_in_block] & valid_s[t];
+            word = mask_s[(t - kWaves) * M + row_in_block] & valid_s[t];
         } else {
             const int left = p.prefix - (t - listed_tiles) * kTileN;
             word = left >= 32 ? 0xffffffffu : ((1u << left) - 1u);
         }
-        if (__ballot(word != 0u) == 0ull) continue;   // none of this wave's queries attends to the tile
-
         // S^T = K_tile . Q^T
         f32x16 s;
 #pragma unroll
@@ -352,23 +392,27 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
             s = MM::mfma(__builtin_bit_cast(Frag, raw), qf[ks], s);
         }
         // V fragments (A operand of O^T += V^T.P^T: rows are head dims) through the
-        // transposing read; issued now so that LDS latency hides behind the softmax
-        VPair vfrag[2][kDTiles];
-        {
-            const int tr_row = (lane & 15) >> 2;                          // key within a group of 4
-            const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);   // head dim within the 32-row tile
+        // transposing read.  The first half of the keys is requested now, so that LDS
+        // latency hides behind the softmax; the second half behind the first MFMAs.
+        const int tr_row = (lane & 15) >> 2;                          // key within a group of 4
+        const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);   // head dim within the 32-row tile
+        auto read_v = [&](VPair (&f)[kDTiles], int kk) {
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk) {
-#pragma unroll
-                for (int dt = 0; dt < kDTiles; ++dt) {
-                    const int col = 32 * dt + tr_col;
-                    const int r0 = 16 * kk + 4 * h + tr_row;      // keys 16kk+4h .. +3
-                    const int r1 = r0 + 8;                         // keys 16kk+8+4h .. +3
-                    vfrag[kk][dt].a = lds_read_tr16(lds_addr(vt + r0 * D + v_chunk<D>(r0, col >> 3) * 8 + (col & 7)));
-                    vfrag[kk][dt].b = lds_read_tr16(lds_addr(vt + r1 * D + v_chunk<D>(r1, col >> 3) * 8 + (col & 7)));
-                }
+            for (int dt = 0; dt < kDTiles; ++dt) {
+                const int col = 32 * dt + tr_col;
+                const int r0 = 16 * kk + 4 * h + tr_row;      // keys 16kk+4h .. +3
+                const int r1 = r0 + 8;                         // keys 16kk+8+4h .. +3
+                f[dt].a = lds_read_tr16(lds_addr(vt + r0 * D + v_chunk<D>(r0, col >> 3) * 8 + (col & 7)));
+                f[dt].b = lds_read_tr16(lds_addr(vt + r1 * D + v_chunk<D>(r1, col >> 3) * 8 + (col & 7)));
             }
-        }
+        };
+        auto tie_v = [&](VPair (&f)[kDTiles]) {
+            lds_wait();
+#pragma unroll
+            for (int dt = 0; dt < kDTiles; ++dt) { lds_tie(f[dt].a); lds_tie(f[dt].b); }
+        };
+        VPair v0[kDTiles], v1[kDTiles];
+        read_v(v0, 0);
         // mask + online softmax; accumulator register r is key 8*(r/4) + 4h + r%4
         const uint32_t wsh = word >> (4 * h);
         float sv[16];
@@ -405,33 +449,37 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
         Frag ph[2], pl[2];
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
+            u32x4 hi4, lo4;
 #pragma unroll
-            for (int e = 0; e < 8; e += 2) {
-                const f32x2 w = {sv[8 * kk + e], sv[8 * kk + e + 1]};
-                const T2 hi = __builtin_convertvector(w, T2);
-                ph[kk][e] = hi[0];
-                ph[kk][e + 1] = hi[1];
-                if (SPLIT) {
-                    const f32x2 rest = w - __builtin_convertvector(hi, f32x2);
-                    const T2 lo = __builtin_convertvector(rest, T2);
-                    pl[kk][e] = lo[0];
-                    pl[kk][e + 1] = lo[1];
-                }
+            for (int e = 0; e < 4; ++e) {
+                const float a = sv[8 * kk + 2 * e], b = sv[8 * kk + 2 * e + 1];
+                const uint32_t hi = MM::pack(a, b);
+                hi4[e] = hi;
+                if (SPLIT) lo4[e] = MM::pack(a - MM::low(hi), b - MM::high(hi));
             }
+            ph[kk] = __builtin_bit_cast(Frag, hi4);
+            if (SPLIT) pl[kk] = __builtin_bit_cast(Frag, lo4);
         }
         // O^T += V_tile^T . P^T ; hi weights of all head-dim tiles first, then lo, so that
         // MFMAs on the same accumulator are several instructions apart
-        wait_lds(vfrag);
+        tie_v(v0);
+        read_v(v1, 1);
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
+        for (int dt = 0; dt < kDTiles; ++dt)
+            o[dt] = MM::mfma(__builtin_bit_cast(Frag, v0[dt]), ph[0], o[dt]);
+        if (SPLIT) {
 #pragma unroll
             for (int dt = 0; dt < kDTiles; ++dt)
-                o[dt] = MM::mfma(__builtin_bit_cast(Frag, vfrag[kk][dt]), ph[kk], o[dt]);
-            if (SPLIT) {
+                o[dt] = MM::mfma(__builtin_bit_cast(Frag, v0[dt]), pl[0], o[dt]);
+        }
+        tie_v(v1);
 #pragma unroll
-                for (int dt = 0; dt < kDTiles; ++dt)
-                    o[dt] = MM::mfma(__builtin_bit_cast(Frag, vfrag[kk][dt]), pl[kk], o[dt]);
-            }
+        for (int dt = 0; dt < kDTiles; ++dt)
+            o[dt] = MM::mfma(__builtin_bit_cast(Frag, v1[dt]), ph[1], o[dt]);
+        if (SPLIT) {
+#pragma unroll
+            for (int dt = 0; dt < kDTiles; ++dt)
+                o[dt] = MM::mfma(__builtin_bit_cast(Frag, v1[dt]), pl[1], o[dt]);
         }
     }
 
@@ -456,12 +504,8 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
                 if (p.out_f32) {
                     *reinterpret_cast<float4*>(static_cast<float*>(p.o) + base + d) = val;
                 } else {
-                    typedef T t4 __attribute__((ext_vector_type(4)));
-                    const T2 lo = __builtin_convertvector((f32x2){val.x, val.y}, T2);
-                    const T2 hi = __builtin_convertvector((f32x2){val.z, val.w}, T2);
-                    t4 packed;
-                    packed[0] = lo[0]; packed[1] = lo[1]; packed[2] = hi[0]; packed[3] = hi[1];
-                    *reinterpret_cast<t4*>(static_cast<T*>(p.o) + base + d) = packed;
+                    const u32x2 packed = {MM::pack(val.x, val.y), MM::pack(val.z, val.w)};
+                    *reinterpret_cast<u32x2*>(static_cast<T*>(p.o) + base + d) = packed;
                 }
             }
         }
@@ -471,7 +515,7 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
 template <bool BF16, int D, int M, bool SPLIT>
 int launch_one(const AttnParams& p, hipStream_t stream) {
     // ring depth: everything in flight at once for short tile lists, else the limit
-    const int tiles = anc_tile_capacity(p.max_anc) + (p.prefix + kTileN - 1) / kTileN;
+    const int tiles = M / 32 + anc_tile_capacity(p.max_anc) + (p.prefix + kTileN - 1) / kTileN;
     int stages = tiles < 2 ? 2 : (tiles > kMaxStages ? kMaxStages : tiles);
     size_t lds = mfma_lds_bytes<D, M>(p.max_anc, stages);
     while (lds > 160 * 1024 && stages > 2) lds = mfma_lds_bytes<D, M>(p.max_anc, --stages);

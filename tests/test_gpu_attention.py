@@ -147,17 +147,21 @@ def test_default_output_dtype_and_bf16_rounding_report():
     assert ((o.cpu().double() - want).abs() <= ulp + 1e-4).all()
 
 
-def test_fast_pv_flag_stays_within_loose_bound():
-    cfg = trees.config(2)
-    a_idx, a_mask, l_idx, max_anc = oracle_inputs(cfg.parent, cfg.block_m)
-    q, k, v = trees.make_qkv(cfg)
-    scale = 1 / math.sqrt(cfg.head_dim)
-    want, _ = dense_oracle(q, k, v, cfg.parent, scale)
+@pytest.mark.parametrize("d", [32, 64, 128])
+@pytest.mark.parametrize("block_m", [32, 64, 128])
+def test_fast_pv_flag_stays_within_loose_bound(d, block_m):
+    # single bf16 rounding of every weight (relative 2^-9 each, weights up to 2^8 before
+    # normalisation): a few 1e-3 of max|v| in practice; a wrong weight would be off by O(1)
+    parent = trees.random_recursive_parents(300, 5 + d + block_m, window=40)
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(parent, block_m)
+    nq = a_idx.shape[0] * block_m
+    q, k, v = rand_qkv(1, 4, nq, nq, d, torch.bfloat16, 3)
+    scale = 1 / math.sqrt(d)
+    want, _ = dense_oracle(q, k, v, parent, scale, nq_pad=nq - 300)
     o = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(), scale,
-                      BLOCK_M=cfg.block_m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32, fast_pv=True)
-    # one bf16 rounding per weight: |err| <= 2^-9 * max|v|, and max|v| of N(0,1) samples is ~5
+                      BLOCK_M=block_m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32, fast_pv=True)
     err = float((o.cpu().double() - want).abs().max())
-    assert err < 2.0 ** -9 * float(v.abs().max()), err
+    assert err < 2.5e-2, err
 
 
 def test_ancestor_slots_with_holes_and_out_of_range_ids_are_skipped():
