@@ -120,11 +120,12 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 // Waits until at most `tiles` tiles' worth of this wave's global->LDS transfers
 // (kPerTile instructions each, retired in order) are still outstanding.
 template <int kPerTile> __device__ __forceinline__ void wait_tiles_outstanding(int tiles) {
-    static_assert((kMaxStages - 2) * kPerTile < 64, "ring too deep for vmcnt");
+    static_assert((kMaxStages - 1) * kPerTile < 64, "ring too deep for vmcnt");
     switch (tiles) {
         case 0: wait_vmcnt<0>(); break;
         case 1: wait_vmcnt<kPerTile>(); break;
-        default: wait_vmcnt<2 * kPerTile>(); break;
+        case 2: wait_vmcnt<2 * kPerTile>(); break;
+        default: wait_vmcnt<3 * kPerTile>(); break;
     }
 }
 
@@ -177,19 +178,30 @@ template <int D> __device__ __forceinline__ int v_chunk(int row, int c) {
     return c ^ (4 * ((row / rpb) % qpr));
 }
 
+// Key-split factor: how many waves share one group of 32 query rows, each taking every
+// KS-th tile with its own running softmax; the partial results are merged through LDS at
+// the end.  Blocks of 64 and 32 rows would otherwise run on 2 or 1 waves.
+constexpr int key_split_for(int block_m) { return block_m >= 128 ? 1 : 2; }
+// Leaf tiles consumed per step (each by a different wave).
+constexpr int leaf_group_for(int block_m) { return block_m >= 64 ? 2 : 1; }
+
 template <bool BF16, int D, int M, bool SPLIT>
-__global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int stages) {
+__global__ __launch_bounds__(M * 2 * key_split_for(M), 2) void attn_mfma_kernel(AttnParams p, int stages) {
     using MM = Mma<BF16>;
     using T = typename MM::elem;
     using T2 = typename MM::elem2;
     using Frag = typename MM::frag;
-    constexpr int kWaves = M / 32;
+    constexpr int kQGroups = M / 32;              // groups of 32 query rows
+    constexpr int kSplit = key_split_for(M);
+    constexpr int kLeafGroup = leaf_group_for(M);
+    constexpr int kWaves = kQGroups * kSplit;
     constexpr int kThreads = kWaves * 64;
     constexpr int kCpr = D / 8;                   // 16-byte chunks per row
     constexpr int kRowsPerDma = 64 / kCpr;        // rows one wave-wide 1 KiB transfer covers
     constexpr int kDmaPerTile = 2 * kTileN / kRowsPerDma;   // K and V transfers of one tile
-    constexpr int kDmaPerWave = kDmaPerTile / kWaves;
-    static_assert(kDmaPerWave * kWaves == kDmaPerTile, "transfers must split evenly over the waves");
+    constexpr int kDmaWaves = kDmaPerTile < kWaves ? kDmaPerTile : kWaves;   // waves that gather
+    constexpr int kDmaPerWave = kDmaPerTile / kDmaWaves;
+    static_assert(kDmaPerWave * kDmaWaves == kDmaPerTile, "transfers must split evenly over the waves");
     constexpr int kRowGroups = (kDmaPerWave + 1) / 2;   // row groups a wave touches per tile
     constexpr int kSteps = D / 16;                // QK^T MFMAs per tile
     constexpr int kDTiles = D / 32;               // 32-row tiles of O^T
@@ -198,7 +210,7 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     T* ring = reinterpret_cast<T*>(smem);                 // [stages][K tile | V tile]
     int* key_s = reinterpret_cast<int*>(ring + stages * 2 * kTileElems);
-    const int cap = kWaves + anc_tile_capacity(p.max_anc);                   // listed tiles
+    const int cap = kQGroups + anc_tile_capacity(p.max_anc);                 // listed tiles
     uint32_t* valid_s = reinterpret_cast<uint32_t*>(key_s + cap * kTileN);   // [cap]
     uint32_t* mask_s = valid_s + cap;                                        // [ancestor tiles][M]
 
@@ -213,10 +225,12 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int qgroup = wave % kQGroups;   // which 32 query rows
+    const int split = wave / kQGroups;    // which share of the tiles
     const int lane = tid & 63;
     const int ql = lane & 31;        // query (column of S^T / O^T) of this lane
     const int h = lane >> 5;         // which half of the rows of the accumulator tile
-    const int row_in_block = wave * 32 + ql;
+    const int row_in_block = qgroup * 32 + ql;
     const int qrow = j * M + row_in_block;
     const bool q_ok = qrow < p.nq;
 
@@ -228,7 +242,7 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
     int n_anc = p.anc_count ? p.anc_count[j] : p.max_anc;
     const int64_t leaf64 = p.leaf_idx[(size_t)j * M + row_in_block];
     const bool leaf_ok = leaf64 >= 0 && leaf64 < p.nk;
-    // Sanitised key lists: the block's M leaf slots (tiles 0 .. kWaves-1), then the
+    // Sanitised key lists: the block's M leaf slots (tiles 0 .. kQGroups-1), then the
     // ancestor slots.  An empty or out-of-range slot is given the row of the first valid
     // key of its tile (row 0 if the tile has none): the transfer count per tile stays
     // fixed, the slot's mask bits are cleared through valid_s, and the data it brings in
@@ -259,20 +273,20 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
         qf[s] = __builtin_bit_cast(Frag, raw);
     }
     n_anc = min(max(n_anc, 0), p.max_anc);
-    const int listed_tiles = kWaves + (n_anc + kTileN - 1) / kTileN;
+    const int listed_tiles = kQGroups + (n_anc + kTileN - 1) / kTileN;
     const int total_tiles = listed_tiles + (p.prefix + kTileN - 1) / kTileN;
-    const int ahead = stages - 1;   // tiles kept in flight beyond the one in use
     __syncthreads();
 
     // ---- gather: HBM -> LDS, 16 bytes per lane, no registers in between --------
     // Transfer g of a tile moves row group g/2 = rows [kRowsPerDma*(g/2), +kRowsPerDma) of K
-    // (g even) or V (g odd); wave w issues transfers [w*kDmaPerWave, +kDmaPerWave).  Lane i
-    // lands at LDS byte 16*i of the transfer, i.e. row i / kCpr, chunk slot i % kCpr, and
-    // fetches the chunk that the XOR swizzle assigns to that slot.  Every wave issues exactly
-    // kDmaPerWave transfers per tile: the vmcnt bookkeeping below counts on it.
+    // (g even) or V (g odd); wave w < kDmaWaves issues transfers [w*kDmaPerWave, +kDmaPerWave).
+    // Lane i lands at LDS byte 16*i of the transfer, i.e. row i / kCpr, chunk slot i % kCpr,
+    // and fetches the chunk that the XOR swizzle assigns to that slot.  Every gathering wave
+    // issues exactly kDmaPerWave transfers per tile: the vmcnt bookkeeping counts on it.
     const int dma_row = lane / kCpr, dma_slot = lane % kCpr;
-    auto issue = [&](int t, int stage) {
-        T* dst_tile = ring + stage * 2 * kTileElems;
+    auto issue = [&](int t, int slot) {
+        if (kDmaWaves < kWaves && wave >= kDmaWaves) return;
+        T* dst_tile = ring + slot * 2 * kTileElems;
         int rows[kRowGroups];
 #pragma unroll
         for (int i = 0; i < kRowGroups; ++i) {
@@ -288,7 +302,7 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
             const int r = u * kRowsPerDma + dma_row;
             const size_t row_off = (size_t)rows[u - (wave * kDmaPerWave) / 2] * D;
             // V of a leaf tile is read row-wise like K (no transposing read), so it takes K's swizzle
-            const T* src = is_v ? vb + row_off + (t < kWaves ? k_chunk<D>(r, dma_slot) : v_chunk<D>(r, dma_slot)) * 8
+            const T* src = is_v ? vb + row_off + (t < kQGroups ? k_chunk<D>(r, dma_slot) : v_chunk<D>(r, dma_slot)) * 8
                                 : kb + row_off + k_chunk<D>(r, dma_slot) * 8;
             __builtin_amdgcn_global_load_lds(
                 (const void __attribute__((address_space(1)))*)src,
@@ -296,8 +310,36 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
                 16, 0, 0);
         }
     };
-    for (int t = 0; t < ahead; ++t)
-        if (t < total_tiles) issue(t, t);
+
+    // Ring bookkeeping, in tiles: `issued` gathers started, `consumed` tiles everyone is done
+    // with; tile i lives in slot i % stages.  begin_step(g) makes tiles [consumed, consumed+g)
+    // usable: wait until at most the gathers issued after them are outstanding (they retire in
+    // order), barrier (everyone's share has landed, everyone is done with the tiles before),
+    // then refill the slots that barrier freed.
+    int issued = 0, issue_slot = 0, consumed = 0, slot = 0;
+    auto refill = [&]() {
+        while (issued < total_tiles && issued < consumed + stages) {
+            issue(issued, issue_slot);
+            ++issued;
+            issue_slot = issue_slot + 1 == stages ? 0 : issue_slot + 1;
+        }
+    };
+    auto begin_step = [&](int g) {
+        wait_tiles_outstanding<kDmaPerWave>(max(issued - consumed - g, 0));
+        __syncthreads();
+        refill();
+    };
+    auto end_step = [&](int g) {
+        consumed += g;
+        slot += g;
+        if (slot >= stages) slot -= stages;
+    };
+    auto tile_ptr = [&](int i) {   // K tile of the i-th tile of the current step; V follows it
+        int sl = slot + i;
+        if (sl >= stages) sl -= stages;
+        return ring + sl * 2 * kTileElems;
+    };
+    refill();
 
     float m_i = -INFINITY, l_i = 0.f;
     f32x16 o[kDTiles];
@@ -306,29 +348,16 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
 #pragma unroll
         for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
 
-    int stage = 0;                      // ring slot of tile t
-    int fill = ahead % stages;          // ring slot the next issued tile goes to (= slot of tile t-1)
-    const T* kt;                        // K tile of the current step; V follows it
-    // Start of step t: tile t has landed once at most the transfers of the tiles issued
-    // after it are outstanding; after the barrier everyone's share of it is in LDS and
-    // everyone is done with tile t-1, whose slot takes the next gather.
-    auto begin_step = [&](int t) {
-        wait_tiles_outstanding<kDmaPerWave>(min(total_tiles - 1 - t, ahead - 1));
-        __syncthreads();
-        if (t + ahead < total_tiles) issue(t + ahead, fill);
-        kt = ring + stage * 2 * kTileElems;
-        fill = stage;
-        stage = stage + 1 == stages ? 0 : stage + 1;
-    };
-
-    // Leaf tile t = the block's own rows 32t .. 32t+31 (reference
+    // Leaf tile i = the block's own rows 32i .. 32i+31 (reference
     // fstattention.py:86-91,104-107): query r sees exactly row r of it, so this is one
-    // dot product per lane pair for wave t, no matrix core; it seeds the running softmax.
-    for (int t = 0; t < kWaves; ++t) {
-        begin_step(t);
-        const T* vt = kt + kTileElems;
-        if (t == wave && __ballot(leaf_ok) != 0ull) {
-            float part = 0.f;
+    // dot product per lane pair for one wave, no matrix core; it seeds that wave's
+    // running softmax.  kLeafGroup leaf tiles are taken per step, by different waves.
+    for (int base = 0; base < kQGroups; base += kLeafGroup) {
+        begin_step(kLeafGroup);
+        if (split == 0 && qgroup >= base && qgroup < base + kLeafGroup && __ballot(leaf_ok) != 0ull) {
+            const T* kt = tile_ptr(qgroup - base);
+            const T* vt = kt + kTileElems;
+            float part[2] = {0.f, 0.f};
             {
                 u32x4 kraw[kSteps];
 #pragma unroll
@@ -343,45 +372,62 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
                     for (int e = 0; e < 4; ++e) {
                         const T2 a = {qf[ks][2 * e], qf[ks][2 * e + 1]};
                         const T2 b = {kf[2 * e], kf[2 * e + 1]};
-                        part = MM::dot2(a, b, part);
+                        part[e & 1] = MM::dot2(a, b, part[e & 1]);
                     }
                 }
             }
-            const float dot = part + __shfl_xor(part, 32);
-            if (leaf_ok) { m_i = dot * p.scale_log2e; l_i = h == 0 ? 1.f : 0.f; }
+            const float half_dot = part[0] + part[1];
+            const float dot = half_dot + __shfl_xor(half_dot, 32);
+            u32x2 vraw[kDTiles][4];
 #pragma unroll
-            for (int dt = 0; dt < kDTiles; ++dt) {
-                u32x2 vraw[4];
+            for (int dt = 0; dt < kDTiles; ++dt)
 #pragma unroll
                 for (int g = 0; g < 4; ++g)   // accumulator rows 8g + 4h .. +3 of tile dt: 4 head dims
-                    vraw[g] = lds_read_b64(lds_addr(vt + ql * D + k_chunk<D>(ql, 4 * dt + g) * 8 + 4 * h));
-                lds_wait();
+                    vraw[dt][g] = lds_read_b64(lds_addr(vt + ql * D + k_chunk<D>(ql, 4 * dt + g) * 8 + 4 * h));
+            lds_wait();
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    lds_tie(vraw[g]);
-                    const uint32_t w0 = vraw[g][0], w1 = vraw[g][1];
-                    o[dt][4 * g + 0] = leaf_ok ? MM::low(w0) : 0.f;
-                    o[dt][4 * g + 1] = leaf_ok ? MM::high(w0) : 0.f;
-                    o[dt][4 * g + 2] = leaf_ok ? MM::low(w1) : 0.f;
-                    o[dt][4 * g + 3] = leaf_ok ? MM::high(w1) : 0.f;
-                }
+            for (int dt = 0; dt < kDTiles; ++dt)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) lds_tie(vraw[dt][g]);
+            if (leaf_ok) {
+                m_i = dot * p.scale_log2e;
+                l_i = h == 0 ? 1.f : 0.f;
+#pragma unroll
+                for (int dt = 0; dt < kDTiles; ++dt)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const uint32_t w0 = vraw[dt][g][0], w1 = vraw[dt][g][1];
+                        o[dt][4 * g + 0] = MM::low(w0);
+                        o[dt][4 * g + 1] = MM::high(w0);
+                        o[dt][4 * g + 2] = MM::low(w1);
+                        o[dt][4 * g + 3] = MM::high(w1);
+                    }
             }
         }
+        end_step(kLeafGroup);
     }
 
-    // Ancestor tiles under the packed tree mask, then the dense shared prefix.  A tile none
-    // of this wave's queries attends to is not skipped: with an all-zero mask word it adds
-    // exact zeros, and a branch-free body spares the accumulators a copy per step.
-    for (int t = kWaves; t < total_tiles; ++t) {
-        begin_step(t);
+    // Ancestor tiles under the packed tree mask, then the dense shared prefix; kSplit tiles
+    // per step, tile consumed+s by the waves of share s.  A tile none of a wave's queries
+    // attends to is not skipped: with an all-zero mask word it adds exact zeros, and a
+    // branch-free body spares the accumulators a copy per step.
+    const int tr_row = (lane & 15) >> 2;                          // key within a group of 4
+    const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);   // head dim within the 32-row tile
+    while (consumed < total_tiles) {
+        begin_step(kSplit);
+        const int t = consumed + split;
+        const T* kt = tile_ptr(split);
         const T* vt = kt + kTileElems;
-        uint32_t word;
+        end_step(kSplit);
+        uint32_t word = 0u;
         if (t < listed_tiles) {
-            word = mask_s[(t - kWaves) * M + row_in_block] & valid_s[t];
-        } else {
+            word = mask_s[(t - kQGroups) * M + row_in_block] & valid_s[t];
+        } else if (t < total_tiles) {
             const int left = p.prefix - (t - listed_tiles) * kTileN;
             word = left >= 32 ? 0xffffffffu : ((1u << left) - 1u);
         }
+        if (kSplit > 1 && t >= total_tiles) continue;   // this share has no tile in the last step
+
         // S^T = K_tile . Q^T
         f32x16 s;
 #pragma unroll
@@ -394,8 +440,6 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
         // V fragments (A operand of O^T += V^T.P^T: rows are head dims) through the
         // transposing read.  The first half of the keys is requested now, so that LDS
         // latency hides behind the softmax; the second half behind the first MFMAs.
-        const int tr_row = (lane & 15) >> 2;                          // key within a group of 4
-        const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);   // head dim within the 32-row tile
         auto read_v = [&](VPair (&f)[kDTiles], int kk) {
 #pragma unroll
             for (int dt = 0; dt < kDTiles; ++dt) {
@@ -483,6 +527,34 @@ __global__ __launch_bounds__(M * 2, 2) void attn_mfma_kernel(AttnParams p, int s
         }
     }
 
+    // ---- merge the shares of a query group (same lanes, same layout) through LDS ----
+    if (kSplit > 1) {
+        __syncthreads();   // the ring is free: every tile has been consumed
+        float* xch = reinterpret_cast<float*>(smem) + (size_t)qgroup * (2 + 16 * kDTiles) * 64;
+        if (split == 1) {
+            xch[lane] = m_i;
+            xch[64 + lane] = l_i;
+#pragma unroll
+            for (int dt = 0; dt < kDTiles; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) xch[(2 + 16 * dt + r) * 64 + lane] = o[dt][r];
+        }
+        __syncthreads();
+        if (split != 0) return;
+        const float m_b = xch[lane], l_b = xch[64 + lane];
+        const float m_new = fmaxf(m_i, m_b);
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        const float a_own = __builtin_amdgcn_exp2f(m_i - m_safe);
+        const float a_oth = __builtin_amdgcn_exp2f(m_b - m_safe);
+        l_i = l_i * a_own + l_b * a_oth;
+        m_i = m_new;
+#pragma unroll
+        for (int dt = 0; dt < kDTiles; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                o[dt][r] = o[dt][r] * a_own + xch[(2 + 16 * dt + r) * 64 + lane] * a_oth;
+    }
+
     // ---- epilogue: normalise, write O once (and the base-2 log-sum-exp) --------
     const float l_tot = l_i + __shfl_xor(l_i, 32);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
@@ -526,7 +598,8 @@ int launch_one(const AttnParams& p, hipStream_t stream) {
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
     const unsigned grid = (unsigned)(kXcds * slices_per_xcd * p.nb);
-    hipLaunchKernelGGL((attn_mfma_kernel<BF16, D, M, SPLIT>), dim3(grid), dim3(M * 2), lds, stream, p, stages);
+    hipLaunchKernelGGL((attn_mfma_kernel<BF16, D, M, SPLIT>), dim3(grid), dim3(M * 2 * key_split_for(M)), lds,
+                       stream, p, stages);
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
 }
