@@ -37,9 +37,11 @@ HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 INFINITY_CACHE_BYTES = 256 << 20
 
-# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/): filled in once measured; None until then.
-MEASURED_TRAFFIC_BYTES = None
+# HBM bytes per launch of the headline kernel (256-node tree, cold buffers) from two
+# rocprofv3 --pmc runs, see profiles/attn_mfma_kernel_cfg2_medusa256_hbm_traffic.txt:
+# FETCH_SIZE 3202 KiB x 2.0 (a plain 256 MiB copy reads 131084 KiB on this counter, i.e. the
+# counter sees half of the read traffic) + WRITE_SIZE 2080 KiB x 1.0 (the copy reads 262144).
+MEASURED_TRAFFIC_BYTES = (3202 * 2 + 2080) * 1024
 
 
 def parse_args():
@@ -49,6 +51,12 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (headline: 2)")
     ap.add_argument("--extra", action="store_true", help="also time configurations 3, 4 and 5")
+    ap.add_argument("--regimes", action="store_true",
+                    help="also time the warm-cache loop, plain stream launches, the Python entry point "
+                         "and the GPU precompute")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
+                    help="instead of the benchmark, run 10 device-to-device copies of MIB MiB "
+                         "(reference point for the FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-graph", action="store_true", help="time plain stream launches only")
     return ap.parse_args()
@@ -241,15 +249,28 @@ def cpu_baseline(wl, budget_s=10.0):
     }
 
 
-def summarize(wl, steps, warmup, use_graph):
+def summarize(wl, steps, warmup, use_graph, regimes):
     cold_wall, cold_ev = time_steps(wl, steps, warmup, rotate=True, use_graph=use_graph)
-    warm_wall, warm_ev = time_steps(wl, steps, warmup, rotate=False, use_graph=use_graph)
-    stream_wall, _ = time_steps(wl, steps, warmup, rotate=True, use_graph=False)
-    return {
-        "cold_us": cold_wall * 1e6, "cold_event_us": cold_ev * 1e6,
-        "warm_us": warm_wall * 1e6, "warm_event_us": warm_ev * 1e6,
-        "stream_launch_us": stream_wall * 1e6,
-    }
+    out = {"cold_us": cold_wall * 1e6, "cold_event_us": cold_ev * 1e6}
+    if regimes:
+        warm_wall, warm_ev = time_steps(wl, steps, warmup, rotate=False, use_graph=use_graph)
+        stream_wall, _ = time_steps(wl, steps, warmup, rotate=True, use_graph=False)
+        out.update({"warm_us": warm_wall * 1e6, "warm_event_us": warm_ev * 1e6,
+                    "stream_launch_us": stream_wall * 1e6})
+    return out
+
+
+def copy_calibration(mib):
+    """10 plain device copies of `mib` MiB: what FETCH_SIZE / WRITE_SIZE read for known traffic."""
+    import torch
+    n = mib << 20
+    src = torch.empty(n, dtype=torch.uint8, device="cuda").fill_(1)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    for _ in range(10):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    print(json.dumps({"copy_bytes": n, "copies": 10}))
 
 
 def main():
@@ -263,6 +284,9 @@ def main():
         print("bench.py: no GPU visible; the hot path has no CPU fallback", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
+    if args.copy_calibration:
+        copy_calibration(args.copy_calibration)
+        return
     use_graph = not args.no_graph
 
     wl = Workload(args.config, sets_bytes=2 * INFINITY_CACHE_BYTES)
@@ -271,7 +295,7 @@ def main():
         print(f"bench.py: parity check failed (max err {max_err:.3e} > {tol})", file=sys.stderr)
         sys.exit(1)
 
-    t = summarize(wl, args.steps, args.warmup, use_graph)
+    t = summarize(wl, args.steps, args.warmup, use_graph, args.regimes)
     step_s = t["cold_us"] * 1e-6
     kernel_s = t["cold_event_us"] * 1e-6
     achieved = wl.kv_bytes / kernel_s / 1e9
@@ -311,13 +335,14 @@ def main():
             "avg_launch_us": round(kernel_s * 1e6, 3),
             "mfma_frac_of_bf16_peak": round(wl.flops / kernel_s / 1e12 / MFMA_BF16_PEAK_TFLOPS, 6),
         },
-        "regimes_us_per_call": {
+    }
+    if args.regimes:
+        result["regimes_us_per_call"] = {
             "cold_graph": round(t["cold_us"], 3), "warm_graph": round(t["warm_us"], 3),
             "cold_stream_launches": round(t["stream_launch_us"], 3),
             "python_api_warm": round(time_python_api(wl, args.steps, args.warmup) * 1e6, 3),
             "gpu_precompute": round(time_precompute(wl) * 1e6, 3),
-        },
-    }
+        }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(wl)
     if args.extra:
@@ -326,7 +351,7 @@ def main():
             w = Workload(idx, sets_bytes=2 * INFINITY_CACHE_BYTES)
             ok_i, err_i, _ = w.check_parity()
             steps = max(20, min(args.steps, 100 if idx == 5 else args.steps))
-            ti = summarize(w, steps, min(args.warmup, 10), use_graph)
+            ti = summarize(w, steps, min(args.warmup, 10), use_graph, True)
             ks = ti["cold_event_us"] * 1e-6
             extra[w.cfg.name] = {
                 "us_per_call_cold": round(ti["cold_us"], 2), "us_per_call_warm": round(ti["warm_us"], 2),

@@ -106,7 +106,7 @@ __host__ __device__ constexpr int anc_tile_capacity(int max_anc) { return (max_a
 template <int D, int M>
 __host__ __device__ constexpr size_t mfma_lds_bytes(int max_anc, int stages) {
     return (size_t)stages * 2 * kTileN * D * 2 +
-           (size_t)(M / 32 + anc_tile_capacity(max_anc)) * (kTileN * 4 + 4) +
+           (size_t)(M / 32 + anc_tile_capacity(max_anc)) * (kTileN * 4 + 4) + 12 +
            (size_t)anc_tile_capacity(max_anc) * M * 4;
 }
 
@@ -212,7 +212,7 @@ __global__ __launch_bounds__(M * 2 * key_split_for(M), 2) void attn_mfma_kernel(
     int* key_s = reinterpret_cast<int*>(ring + stages * 2 * kTileElems);
     const int cap = kQGroups + anc_tile_capacity(p.max_anc);                 // listed tiles
     uint32_t* valid_s = reinterpret_cast<uint32_t*>(key_s + cap * kTileN);   // [cap]
-    uint32_t* mask_s = valid_s + cap;                                        // [ancestor tiles][M]
+    uint32_t* mask_s = valid_s + ((cap + 3) & ~3);                           // [ancestor tiles][M], 16-byte aligned
 
     // Workgroup -> (slice, block): consecutive workgroup ids rotate over the 8
     // XCDs, so give every XCD whole (batch, head) slices; all query blocks of a
@@ -242,26 +242,48 @@ __global__ __launch_bounds__(M * 2 * key_split_for(M), 2) void attn_mfma_kernel(
     int n_anc = p.anc_count ? p.anc_count[j] : p.max_anc;
     const int64_t leaf64 = p.leaf_idx[(size_t)j * M + row_in_block];
     const bool leaf_ok = leaf64 >= 0 && leaf64 < p.nk;
+    // This block's mask words go to LDS as they are: a straight global->LDS copy, 16 bytes
+    // per lane, the 1 KiB pieces dealt round-robin to the waves.
+    {
+        const int mask_bytes = p.mask_words * M * 4;   // multiple of 128
+        const char* src = reinterpret_cast<const char*>(p.mask_bits) + (size_t)j * mask_bytes;
+        for (int piece = wave; piece * 1024 < mask_bytes; piece += kWaves) {
+            if (piece * 1024 + lane * 16 < mask_bytes)
+                __builtin_amdgcn_global_load_lds(
+                    (const void __attribute__((address_space(1)))*)(src + piece * 1024 + lane * 16),
+                    (void __attribute__((address_space(3)))*)(reinterpret_cast<char*>(mask_s) + piece * 1024),
+                    16, 0, 0);
+        }
+    }
     // Sanitised key lists: the block's M leaf slots (tiles 0 .. kQGroups-1), then the
     // ancestor slots.  An empty or out-of-range slot is given the row of the first valid
     // key of its tile (row 0 if the tile has none): the transfer count per tile stays
     // fixed, the slot's mask bits are cleared through valid_s, and the data it brings in
-    // is data the tile holds anyway.
-    for (int c = tid; c < cap * kTileN; c += kThreads) {
-        int64_t idx = -1;
-        if (c < M) idx = p.leaf_idx[(size_t)j * M + c];
-        else if (c - M < p.max_anc) idx = p.ancestor_idx[(size_t)j * p.max_anc + (c - M)];
-        const bool ok = idx >= 0 && idx < p.nk;
-        const uint64_t vote = __ballot(ok);
-        const uint32_t mine = (uint32_t)(vote >> (lane & 32));
-        const int first = mine ? (lane & 32) + __ffs(mine) - 1 : lane;
-        const int fallback = __shfl(ok ? (int)idx : 0, first);
-        key_s[c] = ok ? (int)idx : fallback;
-        if ((lane & 31) == 0) valid_s[c >> 5] = mine;
-    }
-    {
-        const uint32_t* src = p.mask_bits + (size_t)j * p.mask_words * M;
-        for (int e = tid; e < p.mask_words * M; e += kThreads) mask_s[e] = src[e];
+    // is data the tile holds anyway.  The ids are requested kKeyBatch at a time before any
+    // is used, so the list costs one memory round trip, not one per pass.
+    constexpr int kKeyBatch = 4;
+    for (int c0 = tid; c0 < cap * kTileN; c0 += kKeyBatch * kThreads) {
+        int64_t ids[kKeyBatch];
+#pragma unroll
+        for (int i = 0; i < kKeyBatch; ++i) {
+            const int c = c0 + i * kThreads;
+            ids[i] = -1;
+            if (c < M) ids[i] = p.leaf_idx[(size_t)j * M + c];
+            else if (c - M < p.max_anc) ids[i] = p.ancestor_idx[(size_t)j * p.max_anc + (c - M)];
+        }
+#pragma unroll
+        for (int i = 0; i < kKeyBatch; ++i) {
+            const int c = c0 + i * kThreads;
+            if (c < cap * kTileN) {
+                const bool ok = ids[i] >= 0 && ids[i] < p.nk;
+                const uint64_t vote = __ballot(ok);
+                const uint32_t mine = (uint32_t)(vote >> (lane & 32));
+                const int first = mine ? (lane & 32) + __ffs(mine) - 1 : lane;
+                const int fallback = __shfl(ok ? (int)ids[i] : 0, first);
+                key_s[c] = ok ? (int)ids[i] : fallback;
+                if ((lane & 31) == 0) valid_s[c >> 5] = mine;
+            }
+        }
     }
     // Q fragments: B operand of S^T = K.Q^T, lane holds Q[q][16s + 8h .. +7].  Requested
     // after the lists so that waiting for the lists does not wait for Q.

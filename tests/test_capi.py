@@ -1,0 +1,87 @@
+"""The C ABI library loads and exports what include/fsta.h declares (no GPU needed)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from fstattention_amd import _lib
+
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(REPO, "include", "fsta.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fsta_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    names = declared_functions()
+    assert "fsta_attention_fwd" in names and "fsta_precompute" in names
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_library_exports_every_declared_symbol():
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.fail(f"{_lib.LIB_PATH} has not been built (python -m fstattention_amd.build)")
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} is declared in fsta.h but not exported"
+
+
+def test_constants_match_header():
+    text = open(HEADER).read()
+    defs = dict(re.findall(r"#define\s+(FSTA_[A-Z_0-9]+)\s+(-?\d+)u?\b", text))
+    assert int(defs["FSTA_ABI_VERSION"]) == _lib.ABI_VERSION
+    assert (int(defs["FSTA_F32"]), int(defs["FSTA_F16"]), int(defs["FSTA_BF16"])) == (_lib.F32, _lib.F16, _lib.BF16)
+    assert (int(defs["FSTA_OK"]), int(defs["FSTA_EINVAL"]), int(defs["FSTA_EUNSUPPORTED"]),
+            int(defs["FSTA_EHIP"])) == (_lib.OK, _lib.EINVAL, _lib.EUNSUPPORTED, _lib.EHIP)
+    assert (int(defs["FSTA_FLAG_FAST_PV"]), int(defs["FSTA_FLAG_GENERIC"])) == (_lib.FLAG_FAST_PV, _lib.FLAG_GENERIC)
+    assert (int(defs["FSTA_PRE_TOO_MANY_ANCESTORS"]), int(defs["FSTA_PRE_BAD_NODE_ID"]),
+            int(defs["FSTA_PRE_BAD_LEVEL"])) == (_lib.PRE_TOO_MANY_ANCESTORS, _lib.PRE_BAD_NODE_ID, _lib.PRE_BAD_LEVEL)
+
+
+def test_argument_validation_happens_before_any_gpu_work():
+    lib = _lib.load()
+    assert lib.fsta_abi_version() == _lib.ABI_VERSION
+    assert lib.fsta_mask_words(1) == 1 and lib.fsta_mask_words(32) == 1 and lib.fsta_mask_words(33) == 2
+    # every call below is rejected on its arguments; nothing is launched
+    bad_dtype = lib.fsta_attention_fwd(None, None, None, None, None, None, None, None, None,
+                                       1, 1, 16, 16, 64, 7, 7, 16, 8, 1, 1.0, 0, None)
+    assert bad_dtype == _lib.EINVAL and b"dtype" in lib.fsta_last_error()
+    bad_dim = lib.fsta_attention_fwd(None, None, None, None, None, None, None, None, None,
+                                     1, 1, 16, 16, 48, _lib.F16, _lib.F16, 16, 8, 1, 1.0, 0, None)
+    assert bad_dim == _lib.EUNSUPPORTED and b"head_dim" in lib.fsta_last_error()
+    short_k = lib.fsta_attention_fwd(None, None, None, None, None, None, None, None, None,
+                                     1, 1, 16, 8, 64, _lib.F16, _lib.F16, 16, 8, 1, 1.0, 0, None)
+    assert short_k == _lib.EINVAL
+    blocks = lib.fsta_attention_fwd(None, None, None, None, None, None, None, None, None,
+                                    1, 1, 40, 40, 64, _lib.F16, _lib.F16, 16, 8, 2, 1.0, 0, None)
+    assert blocks == _lib.EINVAL and b"num_blocks" in lib.fsta_last_error()
+    null_ptr = lib.fsta_attention_fwd(None, None, None, None, None, None, None, None, None,
+                                      1, 1, 16, 16, 64, _lib.F16, _lib.F16, 16, 8, 1, 1.0, 0, None)
+    assert null_ptr == _lib.EINVAL and b"null" in lib.fsta_last_error()
+    assert lib.fsta_precompute(None, None, 10, 0, 4, 4, 0, None, None, None, None, None, None, None) == _lib.EINVAL
+    assert lib.fsta_precompute(None, None, 0, 1, 4, 4, 0, None, None, None, None, None, None, None) == _lib.OK
+    assert lib.fsta_pack_mask(None, None, 0, 16, 8, None, None, None) == _lib.OK
+    assert lib.fsta_pack_mask(None, None, 2, 16, 0, None, None, None) == _lib.EINVAL
+    assert lib.fsta_lineage_from_parents(None, 5, 0, None, None, None, None) == _lib.EINVAL
+    with pytest.raises(_lib.FstaError):
+        _lib.check(_lib.EINVAL)
+
+
+def test_python_entry_points_refuse_to_run_without_a_gpu_path():
+    import torch
+    from fstattention_amd import create_fst_attention_kernel_inputs, fst_attention, trees
+    q = torch.zeros(1, 1, 16, 16, dtype=torch.float16)
+    idx = torch.full((1, 8), -1, dtype=torch.int64)
+    mask = torch.zeros(1, 16, 8, dtype=torch.bool)
+    leaf = torch.arange(16).view(1, 16)
+    with pytest.raises(ValueError, match="GPU"):
+        fst_attention(q, q, q, idx, mask, leaf, 1.0, BLOCK_M=16, MAX_ANCESTORS=8)
+    if not torch.cuda.is_available():
+        lineage, level = trees.lineage_from_parents([-1, 0, 1])
+        with pytest.raises(RuntimeError, match="GPU"):
+            create_fst_attention_kernel_inputs(lineage, level, 4, 4)
