@@ -479,17 +479,20 @@ __global__ __launch_bounds__(M * 2 * key_split_for(M), 2) void attn_mfma_kernel(
         };
         VPair v0[kDTiles], v1[kDTiles];
         read_v(v0, 0);
-        // mask + online softmax; accumulator register r is key 8*(r/4) + 4h + r%4
+        // mask + online softmax; accumulator register r is key 8*(r/4) + 4h + r%4.  The
+        // maximum is taken over the raw scores (the scale is positive here, the launcher sends
+        // other scales to the scalar kernel) and the scale rides in the FMA under the exp2.
         const uint32_t wsh = word >> (4 * h);
         float sv[16];
-        float mx = -INFINITY;
+        float mx_raw = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const bool on = (wsh >> (8 * (r / 4) + (r % 4))) & 1u;
-            sv[r] = on ? s[r] * p.scale_log2e : -INFINITY;
-            mx = fmaxf(mx, sv[r]);
+            sv[r] = on ? s[r] : -INFINITY;
+            mx_raw = fmaxf(mx_raw, sv[r]);
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        mx_raw = fmaxf(mx_raw, __shfl_xor(mx_raw, 32));
+        const float mx = mx_raw * p.scale_log2e;
         // Raise the running maximum only for rows that would otherwise produce a weight
         // above 2^kRescaleSlack (always when the row had no key so far); rare after the
         // first tiles, so the rescale of the accumulators is a wave-uniform branch.
@@ -503,11 +506,11 @@ __global__ __launch_bounds__(M * 2 * key_split_for(M), 2) void attn_mfma_kernel(
 #pragma unroll
                 for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
         }
-        const float m_safe = m_i == -INFINITY ? 0.f : m_i;
+        const float neg_m = m_i == -INFINITY ? 0.f : -m_i;
         float rowsum = 0.f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            sv[r] = __builtin_amdgcn_exp2f(sv[r] - m_safe);
+            sv[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[r], p.scale_log2e, neg_m));
             rowsum += sv[r];
         }
         l_i += rowsum;

@@ -67,7 +67,8 @@ extern "C" int fsta_attention_fwd(const void* q, const void* k, const void* v, v
     p.scale_log2e = sm_scale * kLog2e;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (!(flags & FSTA_FLAG_GENERIC) && mfma_supported(dtype, head_dim, block_m))
+    // the matrix-core kernel takes row maxima before scaling, which needs a positive scale
+    if (!(flags & FSTA_FLAG_GENERIC) && sm_scale > 0.f && mfma_supported(dtype, head_dim, block_m))
         return launch_attention_mfma(p, dtype, head_dim, (flags & FSTA_FLAG_FAST_PV) != 0, s);
     return launch_attention_generic(p, dtype, head_dim, s);
 }

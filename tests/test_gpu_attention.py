@@ -103,6 +103,13 @@ def test_reference_test_shape_with_and_without_prefix():
         assert_close(o32, want, torch.float16, f"reference shape prefix={prefix}")
 
 
+@pytest.mark.parametrize("scale", [-0.3, 0.0])
+def test_non_positive_scale(scale):
+    parent = trees.random_recursive_parents(128, 77, window=32)
+    for dtype in (torch.float32, torch.bfloat16):
+        run_tree(parent, 64, 1, 2, 64, dtype, 13, scale=scale)
+
+
 def test_ragged_query_count():
     # nq not a multiple of block_m: rows past nq are neither read nor written
     parent = trees.random_recursive_parents(100, 3)
