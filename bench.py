@@ -325,7 +325,7 @@ def main():
         "parity": {"max_abs_err_vs_oracle": max_err, "tol": tol, "ok": ok},
         "roofline": {
             "bound": "hbm",
-            "kernel": "attn_mfma_kernel<bf16, D=128, M=64, split P>" if args.config == 2 else "attn_mfma_kernel",
+            "kernel": "attn_mfma16_kernel<bf16, D=128, M=64, split P>" if args.config == 2 else "attn_mfma16_kernel",
             "achieved": round(achieved, 2),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",

@@ -9,7 +9,7 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libfsta.so"
 
 F32, F16, BF16 = 0, 1, 2
 OK, EINVAL, EUNSUPPORTED, EHIP = 0, -1, -2, -3
-FLAG_FAST_PV, FLAG_GENERIC = 1, 2
+FLAG_FAST_PV, FLAG_GENERIC, FLAG_WIDE_WAVES = 1, 2, 4
 PRE_TOO_MANY_ANCESTORS, PRE_BAD_NODE_ID, PRE_BAD_LEVEL = 1, 2, 4
 ABI_VERSION = 1
 

@@ -80,7 +80,8 @@ def _packed_for(ancestor_idx: torch.Tensor, ancestor_mask) -> PackedTreeMask:
 
 def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
                   BLOCK_M=128, MAX_ANCESTORS=64, *, out_dtype: Optional[torch.dtype] = None,
-                  return_lse: bool = False, fast_pv: bool = False, generic: bool = False):
+                  return_lse: bool = False, fast_pv: bool = False, generic: bool = False,
+                  wide_waves: bool = False):
     """Fused sparse tree attention forward (reference ``fstattention.py:153-181``).
 
     ``q [Z,H,Nq,D]``, ``k,v [Z,H,Nk,D]`` (``Nk - Nq`` leading rows are a dense
@@ -92,8 +93,9 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
     Beyond the reference: ``out_dtype=torch.float32`` keeps the output
     unrounded, ``return_lse`` also returns the base-2 log-sum-exp ``[Z*H, Nq]``
     the reference computes and drops (``fstattention.py:139-141,181``),
-    ``fast_pv`` trades accuracy of the bf16 weights for matrix-core time, and
-    ``generic`` forces the scalar kernel.  Inputs the reference silently
+    ``fast_pv`` trades accuracy of the bf16 weights for matrix-core time,
+    ``generic`` forces the scalar kernel and ``wide_waves`` the matrix-core variant
+    with 32 instead of 16 query rows per wave.  Inputs the reference silently
     mis-handles raise ``ValueError`` here (non-contiguous tensors, index
     tensors whose shapes do not match ``BLOCK_M`` / ``MAX_ANCESTORS``).
     """
@@ -143,7 +145,8 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
     packed = _packed_for(ancestor_idx, ancestor_mask)
     o = torch.empty(q.shape, dtype=out_dtype, device=q.device)
     lse = torch.empty((Z * H, Nq), device=q.device, dtype=torch.float32)
-    flags = (_lib.FLAG_FAST_PV if fast_pv else 0) | (_lib.FLAG_GENERIC if generic else 0)
+    flags = (_lib.FLAG_FAST_PV if fast_pv else 0) | (_lib.FLAG_GENERIC if generic else 0) | \
+        (_lib.FLAG_WIDE_WAVES if wide_waves else 0)
     with torch.cuda.device(q.device):
         _lib.check(lib.fsta_attention_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),

@@ -23,6 +23,7 @@ SOURCES = [
     "fsta_precompute.hip",
     "fsta_attention_generic.hip",
     "fsta_attention_mfma.hip",
+    "fsta_attention_mfma16.hip",
 ]
 
 # packed-fp32 VALU forms are switched off for device code on purpose

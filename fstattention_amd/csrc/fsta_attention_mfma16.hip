@@ -1,0 +1,506 @@
+// Matrix-core tree attention kernel for gfx950, 16 query rows per wave
+// (v_mfma_f32_16x16x32): bf16 / fp16, head_dim 32/64/128, query blocks of 32/64/128 rows.
+//
+// Same structure as the 32-rows-per-wave kernel (tile list [leaf tiles | ancestor tiles |
+// prefix tiles], K/V gathered straight into an LDS ring, transposed products S^T = K.Q^T and
+// O^T += V^T.P^T, base-2 online softmax in the accumulator layout), but a wave keeps only 16
+// query rows: 32 accumulator registers for O^T instead of 64 and 16 for Q instead of 32.  The
+// kernel fits in 128 VGPRs, so four waves share a SIMD and cover each other's waits
+// (gathers, LDS, the serial MFMA -> softmax -> MFMA chain of one tile); the price is that every
+// K/V fragment is read from LDS by twice as many waves.
+//
+// Layouts of v_mfma_f32_16x16x32 (lane = 16*g + i): A holds row i, k = 8g .. 8g+7; B holds
+// k = 8g .. 8g+7, column i; C holds rows 4g .. 4g+3 of column i.  With S^T the column is the
+// query, so a lane owns keys 4g .. 4g+3 of each 16-key half of a tile for ONE query, and the
+// 8 weights it ends up with are exactly its 8 k-slots of the B operand of O^T += V^T.P^T.
+#include "fsta_mfma_common.h"
+
+namespace fsta {
+namespace {
+
+using namespace mfma;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mfma16(f16x8 a, f16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+// Waves that share one group of 16 query rows, each taking every KS-th tile (merged at the end).
+constexpr int key_split16_for(int block_m) { return block_m >= 128 ? 1 : 2; }
+constexpr int leaf_group16_for(int block_m) { return block_m >= 64 ? 2 : 1; }
+
+// V tile swizzle for the transposing read of this kernel: one read instruction touches 16
+// consecutive rows x 32 bytes, so 32-byte granules are XORed with the row.
+template <int D> __device__ __forceinline__ int v16_chunk(int row, int c) {
+    constexpr int gpr = D / 16, rpb = 8 / gpr;   // granules per row, rows per 256 bytes
+    return c ^ (2 * ((row / rpb) % gpr));
+}
+
+template <int D, int M>
+__host__ __device__ constexpr size_t mfma16_lds_bytes(int max_anc, int stages) {
+    return (size_t)stages * 2 * kTileN * D * 2 +
+           (size_t)(M / 32 + anc_tile_capacity(max_anc)) * (kTileN * 4 + 4) + 12 +
+           (size_t)anc_tile_capacity(max_anc) * M * 4;
+}
+
+template <bool BF16, int D, int M, bool SPLIT>
+__global__ __launch_bounds__(M * 4 * key_split16_for(M), 4) void attn_mfma16_kernel(AttnParams p, int stages) {
+    using MM = Mma<BF16>;
+    using T = typename MM::elem;
+    using T2 = typename MM::elem2;
+    using Frag = typename MM::frag;
+    constexpr int kQGroups = M / 16;              // groups of 16 query rows
+    constexpr int kLeafTiles = M / 32;            // 32-row tiles holding the block's own rows
+    constexpr int kSplit = key_split16_for(M);
+    constexpr int kLeafGroup = leaf_group16_for(M);
+    constexpr int kWaves = kQGroups * kSplit;
+    constexpr int kThreads = kWaves * 64;
+    constexpr int kCpr = D / 8;                   // 16-byte chunks per row
+    constexpr int kRowsPerDma = 64 / kCpr;        // rows one wave-wide 1 KiB transfer covers
+    constexpr int kDmaPerTile = 2 * kTileN / kRowsPerDma;   // K and V transfers of one tile
+    constexpr int kDmaWaves = kDmaPerTile < kWaves ? kDmaPerTile : kWaves;   // waves that gather
+    constexpr int kDmaPerWave = kDmaPerTile / kDmaWaves;
+    static_assert(kDmaPerWave * kDmaWaves == kDmaPerTile, "transfers must split evenly over the waves");
+    constexpr int kRowGroups = (kDmaPerWave + 1) / 2;   // row groups a wave touches per tile
+    constexpr int kSteps = D / 32;                // MFMAs per 16-key half of S^T
+    constexpr int kDTiles = D / 16;               // 16-row tiles of O^T
+    constexpr int kTileElems = kTileN * D;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    T* ring = reinterpret_cast<T*>(smem);                 // [stages][K tile | V tile]
+    int* key_s = reinterpret_cast<int*>(ring + stages * 2 * kTileElems);
+    const int cap = kLeafTiles + anc_tile_capacity(p.max_anc);               // listed tiles
+    uint32_t* valid_s = reinterpret_cast<uint32_t*>(key_s + cap * kTileN);   // [cap]
+    uint32_t* mask_s = valid_s + ((cap + 3) & ~3);                           // [ancestor tiles][M], 16-byte aligned
+
+    // Workgroup -> (slice, block), XCD-aware: every XCD gets whole (batch, head) slices, so all
+    // query blocks of a slice share one L2 for the K/V rows they have in common.
+    const int xcd = blockIdx.x % kXcds;
+    const int within = blockIdx.x / kXcds;
+    const int hz = (within / p.nb) * kXcds + xcd;
+    const int j = within % p.nb;
+    if (hz >= p.heads_total) return;
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int qgroup = wave % kQGroups;   // which 16 query rows
+    const int split = wave / kQGroups;    // which share of the tiles
+    const int lane = tid & 63;
+    const int ql = lane & 15;        // query (column of S^T / O^T) of this lane
+    const int g = lane >> 4;         // which quarter of the rows of an accumulator tile
+    const int row_in_block = qgroup * 16 + ql;
+    const int qrow = j * M + row_in_block;
+    const bool q_ok = qrow < p.nq;
+
+    const T* qb = static_cast<const T*>(p.q) + (size_t)hz * p.nq * D;
+    const T* kb = static_cast<const T*>(p.k) + (size_t)hz * p.nk * D;
+    const T* vb = static_cast<const T*>(p.v) + (size_t)hz * p.nk * D;
+
+    // ---- block metadata: the loads nothing else depends on go out first --------
+    int n_anc = p.anc_count ? p.anc_count[j] : p.max_anc;
+    const int64_t leaf64 = p.leaf_idx[(size_t)j * M + row_in_block];
+    const bool leaf_ok = leaf64 >= 0 && leaf64 < p.nk;
+    // mask words: straight global->LDS copy, 16 bytes per lane, 1 KiB pieces dealt to the waves
+    {
+        const int mask_bytes = p.mask_words * M * 4;   // multiple of 128
+        const char* src = reinterpret_cast<const char*>(p.mask_bits) + (size_t)j * mask_bytes;
+        for (int piece = wave; piece * 1024 < mask_bytes; piece += kWaves) {
+            if (piece * 1024 + lane * 16 < mask_bytes)
+                __builtin_amdgcn_global_load_lds(
+                    (const void __attribute__((address_space(1)))*)(src + piece * 1024 + lane * 16),
+                    (void __attribute__((address_space(3)))*)(reinterpret_cast<char*>(mask_s) + piece * 1024),
+                    16, 0, 0);
+        }
+    }
+    // Sanitised key lists: the block's M leaf slots (tiles 0 .. kLeafTiles-1), then the ancestor
+    // slots.  An empty or out-of-range slot is given the row of the first valid key of its tile
+    // (row 0 if the tile has none): the transfer count per tile stays fixed, the slot's mask
+    // bits are cleared through valid_s, and the data it brings in is data the tile holds anyway.
+    constexpr int kKeyBatch = 2;
+    for (int c0 = tid; c0 < cap * kTileN; c0 += kKeyBatch * kThreads) {
+        int64_t ids[kKeyBatch];
+#pragma unroll
+        for (int i = 0; i < kKeyBatch; ++i) {
+            const int c = c0 + i * kThreads;
+            ids[i] = -1;
+            if (c < M) ids[i] = p.leaf_idx[(size_t)j * M + c];
+            else if (c - M < p.max_anc) ids[i] = p.ancestor_idx[(size_t)j * p.max_anc + (c - M)];
+        }
+#pragma unroll
+        for (int i = 0; i < kKeyBatch; ++i) {
+            const int c = c0 + i * kThreads;
+            if (c < cap * kTileN) {
+                const bool ok = ids[i] >= 0 && ids[i] < p.nk;
+                const uint64_t vote = __ballot(ok);
+                const uint32_t mine = (uint32_t)(vote >> (lane & 32));
+                const int first = mine ? (lane & 32) + __ffs(mine) - 1 : lane;
+                const int fallback = __shfl(ok ? (int)ids[i] : 0, first);
+                key_s[c] = ok ? (int)ids[i] : fallback;
+                if ((lane & 31) == 0) valid_s[c >> 5] = mine;
+            }
+        }
+    }
+    // Q fragments: B operand of S^T = K.Q^T, lane holds Q[q][32s + 8g .. +7]
+    Frag qf[kSteps];
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) {
+        u32x4 raw = {0u, 0u, 0u, 0u};
+        if (q_ok) raw = *reinterpret_cast<const u32x4*>(qb + (size_t)qrow * D + 32 * s + 8 * g);
+        qf[s] = __builtin_bit_cast(Frag, raw);
+    }
+    n_anc = min(max(n_anc, 0), p.max_anc);
+    const int listed_tiles = kLeafTiles + (n_anc + kTileN - 1) / kTileN;
+    const int total_tiles = listed_tiles + (p.prefix + kTileN - 1) / kTileN;
+    __syncthreads();
+
+    // ---- gather: HBM -> LDS, 16 bytes per lane, no registers in between --------
+    // Transfer t2 of a tile moves row group t2/2 = rows [kRowsPerDma*(t2/2), +kRowsPerDma) of K
+    // (t2 even) or V (t2 odd); wave w < kDmaWaves issues transfers [w*kDmaPerWave, +kDmaPerWave).
+    // Lane i lands at LDS byte 16*i of the transfer, i.e. row i / kCpr, chunk slot i % kCpr, and
+    // fetches the chunk that the XOR swizzle assigns to that slot.  Every gathering wave issues
+    // exactly kDmaPerWave transfers per tile: the vmcnt bookkeeping counts on it.
+    const int dma_row = lane / kCpr, dma_slot = lane % kCpr;
+    auto issue = [&](int t, int slot) {
+        if (kDmaWaves < kWaves && wave >= kDmaWaves) return;
+        T* dst_tile = ring + slot * 2 * kTileElems;
+        int rows[kRowGroups];
+#pragma unroll
+        for (int i = 0; i < kRowGroups; ++i) {
+            const int r = ((wave * kDmaPerWave) / 2 + i) * kRowsPerDma + dma_row;
+            if (t < listed_tiles) rows[i] = key_s[t * kTileN + r];
+            else rows[i] = min((t - listed_tiles) * kTileN + r, p.prefix - 1);
+        }
+#pragma unroll
+        for (int i = 0; i < kDmaPerWave; ++i) {
+            const int t2 = wave * kDmaPerWave + i;
+            const int u = t2 >> 1;
+            const bool is_v = t2 & 1;
+            const int r = u * kRowsPerDma + dma_row;
+            const size_t row_off = (size_t)rows[u - (wave * kDmaPerWave) / 2] * D;
+            // V of a leaf tile is read row-wise like K (no transposing read), so it takes K's swizzle
+            const T* src = is_v ? vb + row_off + (t < kLeafTiles ? k_chunk<D>(r, dma_slot) : v16_chunk<D>(r, dma_slot)) * 8
+                                : kb + row_off + k_chunk<D>(r, dma_slot) * 8;
+            __builtin_amdgcn_global_load_lds(
+                (const void __attribute__((address_space(1)))*)src,
+                (void __attribute__((address_space(3)))*)(dst_tile + (is_v ? kTileElems : 0) + u * 512),
+                16, 0, 0);
+        }
+    };
+
+    // Ring bookkeeping, in tiles: `issued` gathers started, `consumed` tiles everyone is done
+    // with; tile i lives in slot i % stages.  begin_step(n) makes tiles [consumed, consumed+n)
+    // usable: wait until at most the gathers issued after them are outstanding (they retire in
+    // order), barrier (everyone's share has landed, everyone is done with the tiles before),
+    // then refill the slots that barrier freed.
+    int issued = 0, issue_slot = 0, consumed = 0, slot = 0;
+    auto refill = [&]() {
+        while (issued < total_tiles && issued < consumed + stages) {
+            issue(issued, issue_slot);
+            ++issued;
+            issue_slot = issue_slot + 1 == stages ? 0 : issue_slot + 1;
+        }
+    };
+    auto begin_step = [&](int n) {
+        wait_tiles_outstanding<kDmaPerWave>(max(issued - consumed - n, 0));
+        __syncthreads();
+        refill();
+    };
+    auto end_step = [&](int n) {
+        consumed += n;
+        slot += n;
+        if (slot >= stages) slot -= stages;
+    };
+    auto tile_ptr = [&](int i) {   // K tile of the i-th tile of the current step; V follows it
+        int sl = slot + i;
+        if (sl >= stages) sl -= stages;
+        return ring + sl * 2 * kTileElems;
+    };
+    refill();
+
+    float m_i = -INFINITY, l_i = 0.f;
+    f32x4 o[kDTiles];
+#pragma unroll
+    for (int dt = 0; dt < kDTiles; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // Leaf tile i = the block's own rows 32i .. 32i+31 (reference fstattention.py:86-91,104-107):
+    // query r sees exactly row r of it.  The two waves owning those rows take one dot product
+    // per query from it on the vector ALU and seed their running softmax with it.
+    for (int base = 0; base < kLeafTiles; base += kLeafGroup) {
+        begin_step(kLeafGroup);
+        const int my_tile = qgroup >> 1;
+        if (split == 0 && my_tile >= base && my_tile < base + kLeafGroup && __ballot(leaf_ok) != 0ull) {
+            const T* kt = tile_ptr(my_tile - base);
+            const T* vt = kt + kTileElems;
+            const int row = (qgroup & 1) * 16 + ql;   // this query's row of the leaf tile
+            float part[2] = {0.f, 0.f};
+            {
+                u32x4 kraw[kSteps];
+#pragma unroll
+                for (int ks = 0; ks < kSteps; ++ks)
+                    kraw[ks] = lds_read_b128(lds_addr(kt + row * D + k_chunk<D>(row, 4 * ks + g) * 8));
+                lds_wait();
+#pragma unroll
+                for (int ks = 0; ks < kSteps; ++ks) {
+                    lds_tie(kraw[ks]);
+                    const Frag kf = __builtin_bit_cast(Frag, kraw[ks]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const T2 a = {qf[ks][2 * e], qf[ks][2 * e + 1]};
+                        const T2 b = {kf[2 * e], kf[2 * e + 1]};
+                        part[e & 1] = MM::dot2(a, b, part[e & 1]);
+                    }
+                }
+            }
+            float dot = part[0] + part[1];
+            dot += __shfl_xor(dot, 16);
+            dot += __shfl_xor(dot, 32);
+            u32x2 vraw[kDTiles];
+#pragma unroll
+            for (int dt = 0; dt < kDTiles; ++dt)   // accumulator rows 4g .. 4g+3 of tile dt: 4 head dims
+                vraw[dt] = lds_read_b64(lds_addr(vt + row * D + k_chunk<D>(row, 2 * dt + (g >> 1)) * 8 + 4 * (g & 1)));
+            lds_wait();
+#pragma unroll
+            for (int dt = 0; dt < kDTiles; ++dt) lds_tie(vraw[dt]);
+            if (leaf_ok) {
+                m_i = dot * p.scale_log2e;
+                l_i = g == 0 ? 1.f : 0.f;
+#pragma unroll
+                for (int dt = 0; dt < kDTiles; ++dt) {
+                    o[dt][0] = MM::low(vraw[dt][0]);
+                    o[dt][1] = MM::high(vraw[dt][0]);
+                    o[dt][2] = MM::low(vraw[dt][1]);
+                    o[dt][3] = MM::high(vraw[dt][1]);
+                }
+            }
+        }
+        end_step(kLeafGroup);
+    }
+
+    // Ancestor tiles under the packed tree mask, then the dense shared prefix; kSplit tiles per
+    // step, tile consumed+s by the waves of share s.  A tile none of a wave's queries attends
+    // to is not skipped: with an all-zero mask word it adds exact zeros, and a branch-free body
+    // spares the accumulators a copy per step.
+    const int tr_row = ql >> 2;         // key within a group of 4
+    const int tr_col = 4 * (ql & 3);    // head dim within the 16-row tile
+    while (consumed < total_tiles) {
+        begin_step(kSplit);
+        const int t = consumed + split;
+        const T* kt = tile_ptr(split);
+        const T* vt = kt + kTileElems;
+        end_step(kSplit);
+        uint32_t word = 0u;
+        if (t < listed_tiles) {
+            word = mask_s[(t - kLeafTiles) * M + row_in_block] & valid_s[t];
+        } else if (t < total_tiles) {
+            const int left = p.prefix - (t - listed_tiles) * kTileN;
+            word = left >= 32 ? 0xffffffffu : ((1u << left) - 1u);
+        }
+        if (kSplit > 1 && t >= total_tiles) continue;   // this share has no tile in the last step
+
+        // S^T = K_tile . Q^T, two halves of 16 keys
+        f32x4 s[2];
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+            s[sub] = f32x4{0.f, 0.f, 0.f, 0.f};
+            const int row = 16 * sub + ql;
+#pragma unroll
+            for (int ks = 0; ks < kSteps; ++ks) {
+                const u32x4 raw = *reinterpret_cast<const u32x4*>(kt + row * D + k_chunk<D>(row, 4 * ks + g) * 8);
+                s[sub] = mfma16(__builtin_bit_cast(Frag, raw), qf[ks], s[sub]);
+            }
+        }
+        // V fragments (A operand of O^T += V^T.P^T: rows are head dims) through the transposing
+        // read: k-slots 8g .. 8g+3 are keys 4g .. 4g+3, k-slots 8g+4 .. 8g+7 keys 16+4g .. 16+4g+3.
+        // Half of the head-dim tiles are requested now (LDS latency hides behind the softmax),
+        // the other half behind the first MFMAs.
+        constexpr int kHalf = kDTiles / 2;
+        auto read_v = [&](VPair (&f)[kHalf], int first_dt) {
+#pragma unroll
+            for (int i = 0; i < kHalf; ++i) {
+                const int col = 16 * (first_dt + i) + tr_col;
+                const int r0 = 4 * g + tr_row;
+                const int r1 = r0 + 16;
+                f[i].a = lds_read_tr16(lds_addr(vt + r0 * D + v16_chunk<D>(r0, col >> 3) * 8 + (col & 7)));
+                f[i].b = lds_read_tr16(lds_addr(vt + r1 * D + v16_chunk<D>(r1, col >> 3) * 8 + (col & 7)));
+            }
+        };
+        auto tie_v = [&](VPair (&f)[kHalf]) {
+            lds_wait();
+#pragma unroll
+            for (int i = 0; i < kHalf; ++i) { lds_tie(f[i].a); lds_tie(f[i].b); }
+        };
+        VPair v0[kHalf], v1[kHalf];
+        read_v(v0, 0);
+        // mask + online softmax; register j of half `sub` is key 16*sub + 4g + j.  The maximum is
+        // taken over the raw scores (the scale is positive here) and the scale rides in the FMA
+        // under the exp2.
+        const uint32_t wsh = word >> (4 * g);
+        float sv[8];
+        float mx_raw = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const bool on = (wsh >> (16 * (r / 4) + (r % 4))) & 1u;
+            sv[r] = on ? s[r / 4][r % 4] : -INFINITY;
+            mx_raw = fmaxf(mx_raw, sv[r]);
+        }
+        mx_raw = fmaxf(mx_raw, __shfl_xor(mx_raw, 16));
+        mx_raw = fmaxf(mx_raw, __shfl_xor(mx_raw, 32));
+        const float mx = mx_raw * p.scale_log2e;
+        // Raise the running maximum only for rows that would otherwise produce a weight above
+        // 2^kRescaleSlack (always when the row had no key so far): a rare wave-uniform branch.
+        const bool raise = mx > m_i + kRescaleSlack || (m_i == -INFINITY && mx > -INFINITY);
+        if (__ballot(raise) != 0ull) {
+            const float alpha = raise ? __builtin_amdgcn_exp2f(m_i - mx) : 1.f;   // exp2(-inf) = 0
+            if (raise) m_i = mx;
+            l_i *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < kDTiles; ++dt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+        }
+        const float neg_m = m_i == -INFINITY ? 0.f : -m_i;
+        float rowsum = 0.f;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            sv[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[r], p.scale_log2e, neg_m));
+            rowsum += sv[r];
+        }
+        l_i += rowsum;
+        // P^T fragment: the 8 weights are this lane's 8 k-slots
+        u32x4 hi4, lo4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float a = sv[2 * e], b = sv[2 * e + 1];
+            const uint32_t hi = MM::pack(a, b);
+            hi4[e] = hi;
+            if (SPLIT) lo4[e] = MM::pack(a - MM::low(hi), b - MM::high(hi));
+        }
+        const Frag ph = __builtin_bit_cast(Frag, hi4);
+        Frag pl;
+        if (SPLIT) pl = __builtin_bit_cast(Frag, lo4);
+        // O^T += V_tile^T . P^T
+        tie_v(v0);
+        read_v(v1, kHalf);
+#pragma unroll
+        for (int i = 0; i < kHalf; ++i) o[i] = mfma16(__builtin_bit_cast(Frag, v0[i]), ph, o[i]);
+        if (SPLIT) {
+#pragma unroll
+            for (int i = 0; i < kHalf; ++i) o[i] = mfma16(__builtin_bit_cast(Frag, v0[i]), pl, o[i]);
+        }
+        tie_v(v1);
+#pragma unroll
+        for (int i = 0; i < kHalf; ++i) o[kHalf + i] = mfma16(__builtin_bit_cast(Frag, v1[i]), ph, o[kHalf + i]);
+        if (SPLIT) {
+#pragma unroll
+            for (int i = 0; i < kHalf; ++i) o[kHalf + i] = mfma16(__builtin_bit_cast(Frag, v1[i]), pl, o[kHalf + i]);
+        }
+    }
+
+    // ---- merge the shares of a query group (same lanes, same layout) through LDS ----
+    if (kSplit > 1) {
+        __syncthreads();   // the ring is free: every tile has been consumed
+        float* xch = reinterpret_cast<float*>(smem) + (size_t)qgroup * (2 + 4 * kDTiles) * 64;
+        if (split == 1) {
+            xch[lane] = m_i;
+            xch[64 + lane] = l_i;
+#pragma unroll
+            for (int dt = 0; dt < kDTiles; ++dt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) xch[(2 + 4 * dt + r) * 64 + lane] = o[dt][r];
+        }
+        __syncthreads();
+        if (split != 0) return;
+        const float m_b = xch[lane], l_b = xch[64 + lane];
+        const float m_new = fmaxf(m_i, m_b);
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        const float a_own = __builtin_amdgcn_exp2f(m_i - m_safe);
+        const float a_oth = __builtin_amdgcn_exp2f(m_b - m_safe);
+        l_i = l_i * a_own + l_b * a_oth;
+        m_i = m_new;
+#pragma unroll
+        for (int dt = 0; dt < kDTiles; ++dt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                o[dt][r] = o[dt][r] * a_own + xch[(2 + 4 * dt + r) * 64 + lane] * a_oth;
+    }
+
+    // ---- epilogue: normalise, write O once (and the base-2 log-sum-exp) --------
+    float l_tot = l_i + __shfl_xor(l_i, 16);
+    l_tot += __shfl_xor(l_tot, 32);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (q_ok) {
+        if (p.lse && g == 0)
+            p.lse[(size_t)hz * p.nq + qrow] = l_tot > 0.f ? m_i + log2f(l_tot) : -INFINITY;
+        const size_t base = ((size_t)hz * p.nq + qrow) * D;
+#pragma unroll
+        for (int dt = 0; dt < kDTiles; ++dt) {
+            // accumulator rows 4g .. 4g+3 of tile dt are 4 consecutive head dims
+            const int d = 16 * dt + 4 * g;
+            float4 val;
+            val.x = o[dt][0] * inv;
+            val.y = o[dt][1] * inv;
+            val.z = o[dt][2] * inv;
+            val.w = o[dt][3] * inv;
+            if (p.out_f32) {
+                *reinterpret_cast<float4*>(static_cast<float*>(p.o) + base + d) = val;
+            } else {
+                const u32x2 packed = {MM::pack(val.x, val.y), MM::pack(val.z, val.w)};
+                *reinterpret_cast<u32x2*>(static_cast<T*>(p.o) + base + d) = packed;
+            }
+        }
+    }
+}
+
+template <bool BF16, int D, int M, bool SPLIT>
+int launch_one(const AttnParams& p, hipStream_t stream) {
+    // ring depth: everything in flight at once for short tile lists, else the limit
+    const int tiles = M / 32 + anc_tile_capacity(p.max_anc) + (p.prefix + kTileN - 1) / kTileN;
+    int stages = tiles < 2 ? 2 : (tiles > kMaxStages ? kMaxStages : tiles);
+    size_t lds = mfma16_lds_bytes<D, M>(p.max_anc, stages);
+    while (lds > 160 * 1024 && stages > 2) lds = mfma16_lds_bytes<D, M>(p.max_anc, --stages);
+    if (lds > 160 * 1024)
+        return fail(FSTA_EUNSUPPORTED, "max_ancestors=%d needs %zu bytes of LDS (limit 163840)", p.max_anc, lds);
+    if (lds > 64 * 1024)
+        FSTA_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_mfma16_kernel<BF16, D, M, SPLIT>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
+    const unsigned grid = (unsigned)(kXcds * slices_per_xcd * p.nb);
+    hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT>), dim3(grid), dim3(M * 4 * key_split16_for(M)), lds,
+                       stream, p, stages);
+    FSTA_HIP_OK(hipGetLastError());
+    return FSTA_OK;
+}
+
+template <bool BF16, int D, bool SPLIT>
+int launch_m(const AttnParams& p, hipStream_t stream) {
+    switch (p.block_m) {
+        case 32: return launch_one<BF16, D, 32, SPLIT>(p, stream);
+        case 64: return launch_one<BF16, D, 64, SPLIT>(p, stream);
+        case 128: return launch_one<BF16, D, 128, SPLIT>(p, stream);
+    }
+    return fail(FSTA_EUNSUPPORTED, "matrix-core kernel: block_m=%d", p.block_m);
+}
+
+template <bool BF16, bool SPLIT>
+int launch_d(const AttnParams& p, int head_dim, hipStream_t stream) {
+    switch (head_dim) {
+        case 32: return launch_m<BF16, 32, SPLIT>(p, stream);
+        case 64: return launch_m<BF16, 64, SPLIT>(p, stream);
+        case 128: return launch_m<BF16, 128, SPLIT>(p, stream);
+    }
+    return fail(FSTA_EUNSUPPORTED, "matrix-core kernel: head_dim=%d", head_dim);
+}
+
+}  // namespace
+
+int launch_attention_mfma16(const AttnParams& p, int dtype, int head_dim, bool fast_pv, hipStream_t stream) {
+    if (dtype == FSTA_F16) return launch_d<false, false>(p, head_dim, stream);
+    if (fast_pv) return launch_d<true, false>(p, head_dim, stream);
+    return launch_d<true, true>(p, head_dim, stream);
+}
+
+}  // namespace fsta

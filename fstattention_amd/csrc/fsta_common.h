@@ -44,6 +44,8 @@ int fail(int code, const char* fmt, ...);
 int launch_attention_generic(const AttnParams& p, int dtype, int head_dim, hipStream_t stream);
 int launch_attention_mfma(const AttnParams& p, int dtype, int head_dim, bool fast_pv,
                           hipStream_t stream);
+int launch_attention_mfma16(const AttnParams& p, int dtype, int head_dim, bool fast_pv,
+                            hipStream_t stream);
 bool mfma_supported(int dtype, int head_dim, int block_m);
 
 // ---- element conversion -------------------------------------------------

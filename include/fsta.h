@@ -38,6 +38,9 @@ extern "C" {
                                   value instead of a hi+lo pair (about 2^-9 relative
                                   error per weight instead of 2^-17)            */
 #define FSTA_FLAG_GENERIC   2u /* force the scalar-ALU kernel (any dtype)      */
+#define FSTA_FLAG_WIDE_WAVES 4u /* matrix-core kernel with 32 query rows per wave
+                                  (32x32x16 MFMA, 2 waves per SIMD) instead of 16
+                                  rows per wave (16x16x32 MFMA, 4 waves per SIMD) */
 
 /* bits of the status word written by fsta_precompute */
 #define FSTA_PRE_TOO_MANY_ANCESTORS 1u /* a block has more than max_ancestors unique ancestors */

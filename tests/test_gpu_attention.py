@@ -19,7 +19,7 @@ pytestmark = pytest.mark.gpu
 
 
 def run_tree(parent, block_m, z, h, d, dtype, seed, prefix=0, generic=False, fast_pv=False,
-             scale=None, check_lse=True):
+             scale=None, check_lse=True, wide_waves=False):
     n = len(parent)
     a_idx, a_mask, l_idx, max_anc = oracle_inputs(parent, block_m)
     nb = a_idx.shape[0]
@@ -31,7 +31,8 @@ def run_tree(parent, block_m, z, h, d, dtype, seed, prefix=0, generic=False, fas
         a_idx, l_idx = shift_for_prefix(a_idx, l_idx, prefix)
     o, lse = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(),
                            scale, BLOCK_M=block_m, MAX_ANCESTORS=max_anc,
-                           out_dtype=torch.float32, return_lse=True, generic=generic, fast_pv=fast_pv)
+                           out_dtype=torch.float32, return_lse=True, generic=generic, fast_pv=fast_pv,
+                           wide_waves=wide_waves)
     assert o.dtype == torch.float32 and o.shape == q.shape
     err = assert_close(o, want, dtype, f"n={n} m={block_m} d={d} {dtype} prefix={prefix}")
     if check_lse:
@@ -55,17 +56,20 @@ def test_config2_medusa256(dtype, generic):
              generic=generic)
 
 
+@pytest.mark.parametrize("wide_waves", [False, True])
 @pytest.mark.parametrize("index", [3, 4])
-def test_config3_4_bf16(index):
+def test_config3_4_bf16(index, wide_waves):
     cfg = trees.config(index)
     run_tree(cfg.parent, cfg.block_m, cfg.batch, cfg.heads, cfg.head_dim, torch.bfloat16,
-             cfg.tensor_seed)
+             cfg.tensor_seed, wide_waves=wide_waves)
 
 
-def test_config5_bf16_head_subset_against_oracle():
+@pytest.mark.parametrize("wide_waves", [False, True])
+def test_config5_bf16_head_subset_against_oracle(wide_waves):
     # full tree and block size, 8 of the 512 (batch, head) slices so the oracle stays small
     cfg = trees.config(5)
-    run_tree(cfg.parent, cfg.block_m, 2, 4, cfg.head_dim, torch.bfloat16, cfg.tensor_seed)
+    run_tree(cfg.parent, cfg.block_m, 2, 4, cfg.head_dim, torch.bfloat16, cfg.tensor_seed,
+             wide_waves=wide_waves)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
@@ -74,6 +78,15 @@ def test_config5_bf16_head_subset_against_oracle():
 def test_shapes_sweep(dtype, d, block_m):
     parent = trees.random_recursive_parents(200, 100 + d + block_m, window=48)
     run_tree(parent, block_m, 1, 3, d, dtype, 7)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("d", [32, 64, 128])
+@pytest.mark.parametrize("block_m", [32, 64, 128])
+@pytest.mark.parametrize("prefix", [0, 40])
+def test_shapes_sweep_wide_wave_variant(dtype, d, block_m, prefix):
+    parent = trees.random_recursive_parents(200, 200 + d + block_m, window=48)
+    run_tree(parent, block_m, 1, 3, d, dtype, 7, prefix=prefix, wide_waves=True)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
