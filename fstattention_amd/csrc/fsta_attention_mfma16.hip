@@ -29,8 +29,6 @@ __device__ __forceinline__ f32x4 mfma16(f16x8 a, f16x8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }
 
-// Waves that share one group of 16 query rows, each taking every KS-th tile (merged at the end).
-constexpr int key_split16_for(int block_m) { return block_m >= 128 ? 1 : 2; }
 constexpr int leaf_group16_for(int block_m) { return block_m >= 64 ? 2 : 1; }
 
 // V tile swizzle for the transposing read of this kernel: one read instruction touches 16
@@ -47,15 +45,17 @@ __host__ __device__ constexpr size_t mfma16_lds_bytes(int max_anc, int stages) {
            (size_t)anc_tile_capacity(max_anc) * M * 4;
 }
 
-template <bool BF16, int D, int M, bool SPLIT>
-__global__ __launch_bounds__(M * 4 * key_split16_for(M), 4) void attn_mfma16_kernel(AttnParams p, int stages) {
+// KS = waves that share one group of 16 query rows, each taking every KS-th tile with its own
+// running softmax (merged through LDS at the end).
+template <bool BF16, int D, int M, bool SPLIT, int KS>
+__global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p, int stages) {
     using MM = Mma<BF16>;
     using T = typename MM::elem;
     using T2 = typename MM::elem2;
     using Frag = typename MM::frag;
     constexpr int kQGroups = M / 16;              // groups of 16 query rows
     constexpr int kLeafTiles = M / 32;            // 32-row tiles holding the block's own rows
-    constexpr int kSplit = key_split16_for(M);
+    constexpr int kSplit = KS;
     constexpr int kLeafGroup = leaf_group16_for(M);
     constexpr int kWaves = kQGroups * kSplit;
     constexpr int kThreads = kWaves * 64;
@@ -455,8 +455,8 @@ __global__ __launch_bounds__(M * 4 * key_split16_for(M), 4) void attn_mfma16_ker
     }
 }
 
-template <bool BF16, int D, int M, bool SPLIT>
-int launch_one(const AttnParams& p, hipStream_t stream) {
+template <bool BF16, int D, int M, bool SPLIT, int KS>
+int launch_ks(const AttnParams& p, hipStream_t stream) {
     // ring depth: everything in flight at once for short tile lists, else the limit
     const int tiles = M / 32 + anc_tile_capacity(p.max_anc) + (p.prefix + kTileN - 1) / kTileN;
     int stages = tiles < 2 ? 2 : (tiles > kMaxStages ? kMaxStages : tiles);
@@ -465,14 +465,25 @@ int launch_one(const AttnParams& p, hipStream_t stream) {
     if (lds > 160 * 1024)
         return fail(FSTA_EUNSUPPORTED, "max_ancestors=%d needs %zu bytes of LDS (limit 163840)", p.max_anc, lds);
     if (lds > 64 * 1024)
-        FSTA_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_mfma16_kernel<BF16, D, M, SPLIT>),
+        FSTA_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_mfma16_kernel<BF16, D, M, SPLIT, KS>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
     const unsigned grid = (unsigned)(kXcds * slices_per_xcd * p.nb);
-    hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT>), dim3(grid), dim3(M * 4 * key_split16_for(M)), lds,
-                       stream, p, stages);
+    hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT, KS>), dim3(grid), dim3(M * 4 * KS), lds, stream, p,
+                       stages);
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
+}
+
+template <bool BF16, int D, int M, bool SPLIT>
+int launch_one(const AttnParams& p, hipStream_t stream) {
+    // Key splitting pays when a wave would otherwise walk several ancestor / prefix tiles on
+    // its own and the block is small (few waves); blocks of 128 rows fill the workgroup anyway.
+    const int work_tiles = anc_tile_capacity(p.max_anc) + (p.prefix + kTileN - 1) / kTileN;
+    if constexpr (M < 128) {
+        if (work_tiles >= 2) return launch_ks<BF16, D, M, SPLIT, 2>(p, stream);
+    }
+    return launch_ks<BF16, D, M, SPLIT, 1>(p, stream);
 }
 
 template <bool BF16, int D, bool SPLIT>
