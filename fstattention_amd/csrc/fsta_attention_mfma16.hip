@@ -284,8 +284,14 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     // step, tile consumed+s by the waves of share s.  A tile none of a wave's queries attends
     // to is not skipped: with an all-zero mask word it adds exact zeros, and a branch-free body
     // spares the accumulators a copy per step.
-    const int tr_row = ql >> 2;         // key within a group of 4
-    const int tr_col = 4 * (ql & 3);    // head dim within the 16-row tile
+    // Byte offsets of this lane's fragments inside a tile.  The XOR swizzles only touch the
+    // chunk bits, so the fragment of K-step ks / head-dim tile dt sits at offset0 ^ (ks << 6)
+    // resp. offset0 ^ (dt << 5), and the rows 16 further down at a fixed distance.
+    constexpr int kHalfTileBytes = 16 * D * 2;   // 16 rows
+    const uint32_t k_lane0 = (uint32_t)(ql * D + k_chunk<D>(ql, g) * 8) * 2;
+    const int tr_r0 = 4 * g + (ql >> 2);   // this lane's key row for the transposing read
+    const int tr_col = 4 * (ql & 3);       // head dim within the 16-row tile
+    const uint32_t v_lane0 = (uint32_t)(tr_r0 * D + v16_chunk<D>(tr_r0, tr_col >> 3) * 8 + (tr_col & 7)) * 2;
     while (consumed < total_tiles) {
         begin_step(kSplit);
         const int t = consumed + split;
@@ -302,14 +308,15 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
         if (kSplit > 1 && t >= total_tiles) continue;   // this share has no tile in the last step
 
         // S^T = K_tile . Q^T, two halves of 16 keys
+        typedef const u32x4 __attribute__((address_space(3))) * lds_u32x4;
+        const uint32_t k_addr0 = lds_addr(kt) + k_lane0;
         f32x4 s[2];
 #pragma unroll
         for (int sub = 0; sub < 2; ++sub) {
             s[sub] = f32x4{0.f, 0.f, 0.f, 0.f};
-            const int row = 16 * sub + ql;
 #pragma unroll
             for (int ks = 0; ks < kSteps; ++ks) {
-                const u32x4 raw = *reinterpret_cast<const u32x4*>(kt + row * D + k_chunk<D>(row, 4 * ks + g) * 8);
+                const u32x4 raw = *(lds_u32x4)(uintptr_t)((k_addr0 ^ (uint32_t)(ks << 6)) + sub * kHalfTileBytes);
                 s[sub] = mfma16(__builtin_bit_cast(Frag, raw), qf[ks], s[sub]);
             }
         }
@@ -318,14 +325,13 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
         // Half of the head-dim tiles are requested now (LDS latency hides behind the softmax),
         // the other half behind the first MFMAs.
         constexpr int kHalf = kDTiles / 2;
+        const uint32_t v_addr0 = lds_addr(vt) + v_lane0;
         auto read_v = [&](VPair (&f)[kHalf], int first_dt) {
 #pragma unroll
             for (int i = 0; i < kHalf; ++i) {
-                const int col = 16 * (first_dt + i) + tr_col;
-                const int r0 = 4 * g + tr_row;
-                const int r1 = r0 + 16;
-                f[i].a = lds_read_tr16(lds_addr(vt + r0 * D + v16_chunk<D>(r0, col >> 3) * 8 + (col & 7)));
-                f[i].b = lds_read_tr16(lds_addr(vt + r1 * D + v16_chunk<D>(r1, col >> 3) * 8 + (col & 7)));
+                const uint32_t addr = v_addr0 ^ (uint32_t)((first_dt + i) << 5);
+                f[i].a = lds_read_tr16(addr);
+                f[i].b = lds_read_tr16_at<kHalfTileBytes>(addr);
             }
         };
         auto tie_v = [&](VPair (&f)[kHalf]) {

@@ -116,6 +116,11 @@ __device__ __forceinline__ s16x4 lds_read_tr16(uint32_t addr) {
     asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(out) : "v"(addr) : "memory");
     return out;
 }
+template <int kOffset> __device__ __forceinline__ s16x4 lds_read_tr16_at(uint32_t addr) {
+    s16x4 out;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(out) : "v"(addr), "n"(kOffset) : "memory");
+    return out;
+}
 __device__ __forceinline__ u32x4 lds_read_b128(uint32_t addr) {
     u32x4 out;
     asm volatile("ds_read_b128 %0, %1" : "=v"(out) : "v"(addr) : "memory");
