@@ -438,26 +438,57 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     float l_tot = l_i + __shfl_xor(l_i, 16);
     l_tot += __shfl_xor(l_tot, 32);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    if (q_ok) {
-        if (p.lse && g == 0)
-            p.lse[(size_t)hz * p.nq + qrow] = l_tot > 0.f ? m_i + log2f(l_tot) : -INFINITY;
-        const size_t base = ((size_t)hz * p.nq + qrow) * D;
+    if (q_ok && p.lse && g == 0)
+        p.lse[(size_t)hz * p.nq + qrow] = l_tot > 0.f ? m_i + log2f(l_tot) : -INFINITY;
+    // In the accumulator layout 16 neighbouring lanes hold 16 different rows of O, which the
+    // memory pipeline would write as 64 separate 8-byte pieces per instruction.  The wave
+    // turns its 16 x D block around in LDS instead (the ring is free by now) and stores whole
+    // rows, 16 bytes per lane.  A float32 output goes in two column halves of the same size.
+    constexpr int kStageStride = D * 2 + 16;     // bytes per staged row (padded against bank conflicts)
+    constexpr int kLanesPerRow = D * 2 / 16;
+    constexpr int kRowsPerStore = 64 / kLanesPerRow;
+    constexpr int kStoreIters = 16 / kRowsPerStore;
+    unsigned char* stage;
+    if (kSplit > 1) {
+        stage = smem + (size_t)qgroup * (2 + 4 * kDTiles) * 64 * 4;   // own exchange area, already read
+    } else {
+        __syncthreads();   // every wave is done with the last tile
+        stage = smem + (size_t)qgroup * 16 * kStageStride;
+    }
+    const int st_row = lane / kLanesPerRow, st_piece = lane % kLanesPerRow;
+    const int first_row = j * M + qgroup * 16;
+    auto flush = [&](unsigned char* dst, size_t pitch) {   // dst: row first_row, first staged column
+#pragma unroll
+        for (int i = 0; i < kStoreIters; ++i) {
+            const int r = i * kRowsPerStore + st_row;
+            const u32x4 val = *reinterpret_cast<const u32x4*>(stage + r * kStageStride + st_piece * 16);
+            if (first_row + r < p.nq) *reinterpret_cast<u32x4*>(dst + r * pitch + st_piece * 16) = val;
+        }
+    };
+    if (p.out_f32) {
+        float* ob = static_cast<float*>(p.o) + ((size_t)hz * p.nq + first_row) * D;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int i = 0; i < kDTiles / 2; ++i) {
+                const int dt = h * (kDTiles / 2) + i;
+                const f32x4 val = {o[dt][0] * inv, o[dt][1] * inv, o[dt][2] * inv, o[dt][3] * inv};
+                *reinterpret_cast<f32x4*>(stage + ql * kStageStride + (16 * i + 4 * g) * 4) = val;
+            }
+            __builtin_amdgcn_wave_barrier();
+            flush(reinterpret_cast<unsigned char*>(ob + h * (D / 2)), (size_t)D * 4);
+            __builtin_amdgcn_wave_barrier();
+        }
+    } else {
+        T* ob = static_cast<T*>(p.o) + ((size_t)hz * p.nq + first_row) * D;
 #pragma unroll
         for (int dt = 0; dt < kDTiles; ++dt) {
             // accumulator rows 4g .. 4g+3 of tile dt are 4 consecutive head dims
-            const int d = 16 * dt + 4 * g;
-            float4 val;
-            val.x = o[dt][0] * inv;
-            val.y = o[dt][1] * inv;
-            val.z = o[dt][2] * inv;
-            val.w = o[dt][3] * inv;
-            if (p.out_f32) {
-                *reinterpret_cast<float4*>(static_cast<float*>(p.o) + base + d) = val;
-            } else {
-                const u32x2 packed = {MM::pack(val.x, val.y), MM::pack(val.z, val.w)};
-                *reinterpret_cast<u32x2*>(static_cast<T*>(p.o) + base + d) = packed;
-            }
+            const u32x2 packed = {MM::pack(o[dt][0] * inv, o[dt][1] * inv), MM::pack(o[dt][2] * inv, o[dt][3] * inv)};
+            *reinterpret_cast<u32x2*>(stage + ql * kStageStride + (16 * dt + 4 * g) * 2) = packed;
         }
+        __builtin_amdgcn_wave_barrier();
+        flush(reinterpret_cast<unsigned char*>(ob), (size_t)D * 2);
     }
 }
 
@@ -468,6 +499,9 @@ int launch_ks(const AttnParams& p, hipStream_t stream) {
     int stages = tiles < 2 ? 2 : (tiles > kMaxStages ? kMaxStages : tiles);
     size_t lds = mfma16_lds_bytes<D, M>(p.max_anc, stages);
     while (lds > 160 * 1024 && stages > 2) lds = mfma16_lds_bytes<D, M>(p.max_anc, --stages);
+    // the epilogue reuses the front of the segment: exchange area of a key split, row staging
+    constexpr size_t kEpilogueBytes = KS > 1 ? (size_t)(M / 16) * (2 + D / 4) * 256 : (size_t)M * (D * 2 + 16);
+    if (lds < kEpilogueBytes) lds = kEpilogueBytes;
     if (lds > 160 * 1024)
         return fail(FSTA_EUNSUPPORTED, "max_ancestors=%d needs %zu bytes of LDS (limit 163840)", p.max_anc, lds);
     if (lds > 64 * 1024)
