@@ -100,6 +100,22 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     const T* kb = static_cast<const T*>(p.k) + (size_t)hz * p.nk * D;
     const T* vb = static_cast<const T*>(p.v) + (size_t)hz * p.nk * D;
 
+    // ---- Q rows of this wave: whole rows straight into LDS (front of the ring, which the
+    // gathers only overwrite after the first barrier), K-tile swizzle; rows past the end of a
+    // ragged last block are read as the last row and never stored
+    const int dma_row = lane / kCpr, dma_slot = lane % kCpr;
+    constexpr int kQDma = 16 / kRowsPerDma;
+    static_assert(kQDma >= 1, "a transfer covers at most the wave's 16 rows");
+    T* qstage = ring + wave * 16 * D;
+#pragma unroll
+    for (int i = 0; i < kQDma; ++i) {
+        const int r = i * kRowsPerDma + dma_row;
+        const int grow = min(j * M + qgroup * 16 + r, p.nq - 1);
+        __builtin_amdgcn_global_load_lds(
+            (const void __attribute__((address_space(1)))*)(qb + (size_t)grow * D + k_chunk<D>(r, dma_slot) * 8),
+            (void __attribute__((address_space(3)))*)(qstage + i * 512), 16, 0, 0);
+    }
+
     // ---- block metadata: the loads nothing else depends on go out first --------
     int n_anc = p.anc_count ? p.anc_count[j] : p.max_anc;
     const int64_t leaf64 = p.leaf_idx[(size_t)j * M + row_in_block];
@@ -144,14 +160,13 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
             }
         }
     }
-    // Q fragments: B operand of S^T = K.Q^T, lane holds Q[q][32s + 8g .. +7]
+    // Q fragments: B operand of S^T = K.Q^T, lane holds Q[q][32s + 8g .. +7].  The key lists
+    // above were loaded after the Q rows, and transfers retire in order.
+    wait_vmcnt<0>();
     Frag qf[kSteps];
 #pragma unroll
-    for (int s = 0; s < kSteps; ++s) {
-        u32x4 raw = {0u, 0u, 0u, 0u};
-        if (q_ok) raw = *reinterpret_cast<const u32x4*>(qb + (size_t)qrow * D + 32 * s + 8 * g);
-        qf[s] = __builtin_bit_cast(Frag, raw);
-    }
+    for (int s = 0; s < kSteps; ++s)
+        qf[s] = __builtin_bit_cast(Frag, *reinterpret_cast<const u32x4*>(qstage + ql * D + k_chunk<D>(ql, 4 * s + g) * 8));
     n_anc = min(max(n_anc, 0), p.max_anc);
     const int listed_tiles = kLeafTiles + (n_anc + kTileN - 1) / kTileN;
     const int total_tiles = listed_tiles + (p.prefix + kTileN - 1) / kTileN;
@@ -163,7 +178,6 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     // Lane i lands at LDS byte 16*i of the transfer, i.e. row i / kCpr, chunk slot i % kCpr, and
     // fetches the chunk that the XOR swizzle assigns to that slot.  Every gathering wave issues
     // exactly kDmaPerWave transfers per tile: the vmcnt bookkeeping counts on it.
-    const int dma_row = lane / kCpr, dma_slot = lane % kCpr;
     auto issue = [&](int t, int slot) {
         if (kDmaWaves < kWaves && wave >= kDmaWaves) return;
         T* dst_tile = ring + slot * 2 * kTileElems;
