@@ -211,7 +211,7 @@ __global__ __launch_bounds__(M * 2 * key_split_for(M), 2) void attn_mfma_kernel(
     };
     auto begin_step = [&](int g) {
         wait_tiles_outstanding<kDmaPerWave>(max(issued - consumed - g, 0));
-        __syncthreads();
+        ring_barrier();
         refill();
     };
     auto end_step = [&](int g) {

@@ -41,14 +41,14 @@ template <int D> __device__ __forceinline__ int v16_chunk(int row, int c) {
 template <int D, int M>
 __host__ __device__ constexpr size_t mfma16_lds_bytes(int max_anc, int stages) {
     return (size_t)stages * 2 * kTileN * D * 2 +
-           (size_t)(M / 32 + anc_tile_capacity(max_anc)) * (kTileN * 4 + 4) + 12 +
+           (size_t)(M / 32 + anc_tile_capacity(max_anc)) * (kTileN * 4 + 4) + 12 + 32 +
            (size_t)anc_tile_capacity(max_anc) * M * 4;
 }
 
 // KS = waves that share one group of 16 query rows, each taking every KS-th tile with its own
 // running softmax (merged through LDS at the end).
 template <bool BF16, int D, int M, bool SPLIT, int KS>
-__global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p, int stages) {
+__global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p, int stages, int early_leaf) {
     using MM = Mma<BF16>;
     using T = typename MM::elem;
     using T2 = typename MM::elem2;
@@ -75,7 +75,8 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     int* key_s = reinterpret_cast<int*>(ring + stages * 2 * kTileElems);
     const int cap = kLeafTiles + anc_tile_capacity(p.max_anc);               // listed tiles
     uint32_t* valid_s = reinterpret_cast<uint32_t*>(key_s + cap * kTileN);   // [cap]
-    uint32_t* mask_s = valid_s + ((cap + 3) & ~3);                           // [ancestor tiles][M], 16-byte aligned
+    uint32_t* spec_s = valid_s + ((cap + 3) & ~3);                           // [8] per-wave flags of the start-up
+    uint32_t* mask_s = spec_s + 8;                                           // [ancestor tiles][M], 16-byte aligned
 
     // Workgroup -> (slice, block), XCD-aware: every XCD gets whole (batch, head) slices, so all
     // query blocks of a slice share one L2 for the K/V rows they have in common.
@@ -94,32 +95,17 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     const int g = lane >> 4;         // which quarter of the rows of an accumulator tile
     const int row_in_block = qgroup * 16 + ql;
     const int qrow = j * M + row_in_block;
-    const bool q_ok = qrow < p.nq;
 
     const T* qb = static_cast<const T*>(p.q) + (size_t)hz * p.nq * D;
     const T* kb = static_cast<const T*>(p.k) + (size_t)hz * p.nk * D;
     const T* vb = static_cast<const T*>(p.v) + (size_t)hz * p.nk * D;
 
-    // ---- Q rows of this wave: whole rows straight into LDS (front of the ring, which the
-    // gathers only overwrite after the first barrier), K-tile swizzle; rows past the end of a
-    // ragged last block are read as the last row and never stored
-    const int dma_row = lane / kCpr, dma_slot = lane % kCpr;
-    constexpr int kQDma = 16 / kRowsPerDma;
-    static_assert(kQDma >= 1, "a transfer covers at most the wave's 16 rows");
-    T* qstage = ring + wave * 16 * D;
-#pragma unroll
-    for (int i = 0; i < kQDma; ++i) {
-        const int r = i * kRowsPerDma + dma_row;
-        const int grow = min(j * M + qgroup * 16 + r, p.nq - 1);
-        __builtin_amdgcn_global_load_lds(
-            (const void __attribute__((address_space(1)))*)(qb + (size_t)grow * D + k_chunk<D>(r, dma_slot) * 8),
-            (void __attribute__((address_space(3)))*)(qstage + i * 512), 16, 0, 0);
-    }
-
-    // ---- block metadata: the loads nothing else depends on go out first --------
+    // ---- start-up: everything that needs no metadata goes out before the metadata is read ----
+    // Loads and transfers retire in issue order, so the order below is also the order of use:
+    // mask words, key lists, Q rows, then the first leaf tiles.  The number of transfers issued
+    // after the key lists is a compile-time constant: the wait for the lists can then leave
+    // exactly those in flight.
     int n_anc = p.anc_count ? p.anc_count[j] : p.max_anc;
-    const int64_t leaf64 = p.leaf_idx[(size_t)j * M + row_in_block];
-    const bool leaf_ok = leaf64 >= 0 && leaf64 < p.nk;
     // mask words: straight global->LDS copy, 16 bytes per lane, 1 KiB pieces dealt to the waves
     {
         const int mask_bytes = p.mask_words * M * 4;   // multiple of 128
@@ -132,45 +118,45 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
                     16, 0, 0);
         }
     }
-    // Sanitised key lists: the block's M leaf slots (tiles 0 .. kLeafTiles-1), then the ancestor
-    // slots.  An empty or out-of-range slot is given the row of the first valid key of its tile
-    // (row 0 if the tile has none): the transfer count per tile stays fixed, the slot's mask
-    // bits are cleared through valid_s, and the data it brings in is data the tile holds anyway.
+    // Key lists: the block's M leaf slots, then its ancestor slots, kKeyBatch per thread and
+    // round.  Slots past the end of the lists re-read the last entry and are blanked below.
     constexpr int kKeyBatch = 2;
-    for (int c0 = tid; c0 < cap * kTileN; c0 += kKeyBatch * kThreads) {
-        int64_t ids[kKeyBatch];
+    auto load_ids = [&](int c0, u32x2 (&raw)[kKeyBatch]) {
 #pragma unroll
         for (int i = 0; i < kKeyBatch; ++i) {
             const int c = c0 + i * kThreads;
-            ids[i] = -1;
-            if (c < M) ids[i] = p.leaf_idx[(size_t)j * M + c];
-            else if (c - M < p.max_anc) ids[i] = p.ancestor_idx[(size_t)j * p.max_anc + (c - M)];
+            const int64_t* src = c < M ? p.leaf_idx + (size_t)j * M + c
+                                       : p.ancestor_idx + (size_t)j * p.max_anc + min(c - M, p.max_anc - 1);
+            raw[i] = global_read_b64(src);
         }
+    };
+    auto ids_of = [&](int c0, u32x2 (&raw)[kKeyBatch], int64_t (&ids)[kKeyBatch]) {
 #pragma unroll
         for (int i = 0; i < kKeyBatch; ++i) {
+            lds_tie(raw[i]);
             const int c = c0 + i * kThreads;
-            if (c < cap * kTileN) {
-                const bool ok = ids[i] >= 0 && ids[i] < p.nk;
-                const uint64_t vote = __ballot(ok);
-                const uint32_t mine = (uint32_t)(vote >> (lane & 32));
-                const int first = mine ? (lane & 32) + __ffs(mine) - 1 : lane;
-                const int fallback = __shfl(ok ? (int)ids[i] : 0, first);
-                key_s[c] = ok ? (int)ids[i] : fallback;
-                if ((lane & 31) == 0) valid_s[c >> 5] = mine;
-            }
+            ids[i] = c - M < p.max_anc ? (int64_t)(((uint64_t)raw[i][1] << 32) | raw[i][0]) : -1;
         }
+    };
+    u32x2 leaf_raw = global_read_b64(p.leaf_idx + (size_t)j * M + row_in_block);
+    u32x2 first_raw[kKeyBatch];
+    load_ids(tid, first_raw);
+    // Q rows of this wave: whole rows straight into LDS, K-tile swizzle, parked in the last ring
+    // slots until the fragments have been read (before the first barrier).  Rows past the end of
+    // a ragged last block are read as the last row and never stored.
+    const int dma_row = lane / kCpr, dma_slot = lane % kCpr;
+    constexpr int kQDma = 16 / kRowsPerDma;
+    static_assert(kQDma >= 1, "a transfer covers at most the wave's 16 rows");
+    constexpr int kQSlots = (kWaves * 16 * D + 2 * kTileElems - 1) / (2 * kTileElems);   // ring slots Q occupies
+    T* qstage = ring + (size_t)stages * 2 * kTileElems - (kWaves - wave) * 16 * D;
+#pragma unroll
+    for (int i = 0; i < kQDma; ++i) {
+        const int r = i * kRowsPerDma + dma_row;
+        const int grow = min(j * M + qgroup * 16 + r, p.nq - 1);
+        __builtin_amdgcn_global_load_lds(
+            (const void __attribute__((address_space(1)))*)(qb + (size_t)grow * D + k_chunk<D>(r, dma_slot) * 8),
+            (void __attribute__((address_space(3)))*)(qstage + i * 512), 16, 0, 0);
     }
-    // Q fragments: B operand of S^T = K.Q^T, lane holds Q[q][32s + 8g .. +7].  The key lists
-    // above were loaded after the Q rows, and transfers retire in order.
-    wait_vmcnt<0>();
-    Frag qf[kSteps];
-#pragma unroll
-    for (int s = 0; s < kSteps; ++s)
-        qf[s] = __builtin_bit_cast(Frag, *reinterpret_cast<const u32x4*>(qstage + ql * D + k_chunk<D>(ql, 4 * s + g) * 8));
-    n_anc = min(max(n_anc, 0), p.max_anc);
-    const int listed_tiles = kLeafTiles + (n_anc + kTileN - 1) / kTileN;
-    const int total_tiles = listed_tiles + (p.prefix + kTileN - 1) / kTileN;
-    __syncthreads();
 
     // ---- gather: HBM -> LDS, 16 bytes per lane, no registers in between --------
     // Transfer t2 of a tile moves row group t2/2 = rows [kRowsPerDma*(t2/2), +kRowsPerDma) of K
@@ -178,16 +164,8 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     // Lane i lands at LDS byte 16*i of the transfer, i.e. row i / kCpr, chunk slot i % kCpr, and
     // fetches the chunk that the XOR swizzle assigns to that slot.  Every gathering wave issues
     // exactly kDmaPerWave transfers per tile: the vmcnt bookkeeping counts on it.
-    auto issue = [&](int t, int slot) {
-        if (kDmaWaves < kWaves && wave >= kDmaWaves) return;
+    auto issue_rows = [&](int t, int slot, const int (&rows)[kRowGroups]) {
         T* dst_tile = ring + slot * 2 * kTileElems;
-        int rows[kRowGroups];
-#pragma unroll
-        for (int i = 0; i < kRowGroups; ++i) {
-            const int r = ((wave * kDmaPerWave) / 2 + i) * kRowsPerDma + dma_row;
-            if (t < listed_tiles) rows[i] = key_s[t * kTileN + r];
-            else rows[i] = min((t - listed_tiles) * kTileN + r, p.prefix - 1);
-        }
 #pragma unroll
         for (int i = 0; i < kDmaPerWave; ++i) {
             const int t2 = wave * kDmaPerWave + i;
@@ -204,13 +182,106 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
                 16, 0, 0);
         }
     };
+    // A valid leaf slot of row r names r's own key (reference utils.py:121-122), so the first
+    // leaf tiles are requested on that assumption, in the ring slots Q does not occupy, while
+    // the lists are still on their way.  Lists that say otherwise are honoured below.
+    // This shortens the start-up chain of a launch whose workgroups all run at once; a launch
+    // with several rounds of workgroups hides that chain anyway and would only pay for the
+    // rows of empty slots, so the launcher asks for it (`early_leaf`) for small grids only.
+    constexpr int kEarlyTiles = kLeafTiles < 2 ? kLeafTiles : 2;   // the launcher provides kQSlots + 2 ring slots
+    const int n_spec = early_leaf ? kEarlyTiles : 0;
+#pragma unroll
+    for (int t = 0; t < kEarlyTiles; ++t) {
+        if (t >= n_spec || (kDmaWaves < kWaves && wave >= kDmaWaves)) break;
+        int rows[kRowGroups];
+#pragma unroll
+        for (int i = 0; i < kRowGroups; ++i)
+            rows[i] = min(p.prefix + j * M + t * kTileN + ((wave * kDmaPerWave) / 2 + i) * kRowsPerDma + dma_row, p.nk - 1);
+        issue_rows(t, t, rows);
+    }
+
+    // Sanitised key lists: the block's M leaf slots (tiles 0 .. kLeafTiles-1), then the ancestor
+    // slots.  An empty or out-of-range slot is given the row of the first valid key of its tile
+    // (row 0 if the tile has none): the transfer count per tile stays fixed, the slot's mask
+    // bits are cleared through valid_s, and the data it brings in is data the tile holds anyway.
+    auto store_keys = [&](int c0, const int64_t (&ids)[kKeyBatch]) {
+#pragma unroll
+        for (int i = 0; i < kKeyBatch; ++i) {
+            const int c = c0 + i * kThreads;
+            if (c < cap * kTileN) {
+                const bool ok = ids[i] >= 0 && ids[i] < p.nk;
+                const uint64_t vote = __ballot(ok);
+                const uint32_t mine = (uint32_t)(vote >> (lane & 32));
+                const int first = mine ? (lane & 32) + __ffs(mine) - 1 : lane;
+                const int fallback = __shfl(ok ? (int)ids[i] : 0, first);
+                lds_write_b32(lds_addr(key_s + c), ok ? (int)ids[i] : fallback);
+                if ((lane & 31) == 0) lds_write_b32(lds_addr(valid_s + (c >> 5)), mine);
+            }
+        }
+    };
+    // first batch and the leaf check: wait for the lists, leave the transfers behind them in flight
+    const bool gathers = !(kDmaWaves < kWaves && wave >= kDmaWaves);
+    if (gathers && n_spec) wait_vmcnt<kQDma + kEarlyTiles * kDmaPerWave>();
+    else wait_vmcnt<kQDma>();
+    int64_t first_ids[kKeyBatch];
+    ids_of(tid, first_raw, first_ids);
+    lds_tie(leaf_raw);
+    const int64_t leaf64 = (int64_t)(((uint64_t)leaf_raw[1] << 32) | leaf_raw[0]);
+    store_keys(tid, first_ids);
+    const bool leaf_ok = leaf64 >= 0 && leaf64 < p.nk;
+    {   // does any valid leaf slot name another row than the one requested above?
+        const bool other = leaf_ok && (row_in_block >> 5) < n_spec && leaf64 != (int64_t)p.prefix + qrow;
+        if (lane == 0) lds_write_b32(lds_addr(spec_s + wave), 0u);
+        if (other) lds_write_b32(lds_addr(spec_s + wave), 1u);
+    }
+    // ... further batches only for very long ancestor lists
+    for (int c0 = tid + kKeyBatch * kThreads; c0 < cap * kTileN; c0 += kKeyBatch * kThreads) {
+        u32x2 raw[kKeyBatch];
+        int64_t ids[kKeyBatch];
+        load_ids(c0, raw);
+        wait_vmcnt<0>();
+        ids_of(c0, raw, ids);
+        store_keys(c0, ids);
+    }
+    // Q fragments: B operand of S^T = K.Q^T, lane holds Q[q][32s + 8g .. +7].  Only the leaf
+    // tiles requested above were issued after the Q rows.
+    wait_tiles_outstanding<kDmaPerWave>(gathers ? n_spec : 0);
+    Frag qf[kSteps];
+    {
+        u32x4 qraw[kSteps];
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s)
+            qraw[s] = lds_read_b128(lds_addr(qstage + ql * D + k_chunk<D>(ql, 4 * s + g) * 8));
+        lds_wait();
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+            lds_tie(qraw[s]);
+            qf[s] = __builtin_bit_cast(Frag, qraw[s]);
+        }
+    }
+    n_anc = min(max(n_anc, 0), p.max_anc);
+    const int listed_tiles = kLeafTiles + (n_anc + kTileN - 1) / kTileN;
+    const int total_tiles = listed_tiles + (p.prefix + kTileN - 1) / kTileN;
+    ring_barrier();
+
+    auto issue = [&](int t, int slot) {
+        if (kDmaWaves < kWaves && wave >= kDmaWaves) return;
+        int rows[kRowGroups];
+#pragma unroll
+        for (int i = 0; i < kRowGroups; ++i) {
+            const int r = ((wave * kDmaPerWave) / 2 + i) * kRowsPerDma + dma_row;
+            if (t < listed_tiles) rows[i] = key_s[t * kTileN + r];
+            else rows[i] = min((t - listed_tiles) * kTileN + r, p.prefix - 1);
+        }
+        issue_rows(t, slot, rows);
+    };
 
     // Ring bookkeeping, in tiles: `issued` gathers started, `consumed` tiles everyone is done
     // with; tile i lives in slot i % stages.  begin_step(n) makes tiles [consumed, consumed+n)
     // usable: wait until at most the gathers issued after them are outstanding (they retire in
     // order), barrier (everyone's share has landed, everyone is done with the tiles before),
     // then refill the slots that barrier freed.
-    int issued = 0, issue_slot = 0, consumed = 0, slot = 0;
+    int issued = n_spec, issue_slot = n_spec, consumed = 0, slot = 0;   // n_spec < stages
     auto refill = [&]() {
         while (issued < total_tiles && issued < consumed + stages) {
             issue(issued, issue_slot);
@@ -220,7 +291,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     };
     auto begin_step = [&](int n) {
         wait_tiles_outstanding<kDmaPerWave>(max(issued - consumed - n, 0));
-        __syncthreads();
+        ring_barrier();
         refill();
     };
     auto end_step = [&](int n) {
@@ -233,6 +304,18 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
         if (sl >= stages) sl -= stages;
         return ring + sl * 2 * kTileElems;
     };
+    {   // a leaf list that names other rows than the ones requested: start the ring over
+        const u32x4 f0 = lds_read_b128(lds_addr(spec_s)), f1 = lds_read_b128(lds_addr(spec_s + 4));
+        lds_wait();
+        u32x4 any = f0 | f1;
+        lds_tie(any);
+        if (__builtin_amdgcn_readfirstlane(any[0] | any[1] | any[2] | any[3]) != 0u) {
+            wait_vmcnt<0>();
+            __syncthreads();
+            issued = 0;
+            issue_slot = 0;
+        }
+    }
     refill();
 
     float m_i = -INFINITY, l_i = 0.f;
@@ -452,8 +535,15 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     float l_tot = l_i + __shfl_xor(l_i, 16);
     l_tot += __shfl_xor(l_tot, 32);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    if (q_ok && p.lse && g == 0)
-        p.lse[(size_t)hz * p.nq + qrow] = l_tot > 0.f ? m_i + log2f(l_tot) : -INFINITY;
+    {
+        // the row number is derived again from an opaque copy: kept from the start-up it would
+        // occupy a register pair through the whole kernel
+        int rib = row_in_block;
+        asm volatile("" : "+v"(rib));
+        const int row = j * M + rib;
+        if (row < p.nq && p.lse && g == 0)
+            p.lse[(size_t)hz * p.nq + row] = l_tot > 0.f ? m_i + log2f(l_tot) : -INFINITY;
+    }
     // In the accumulator layout 16 neighbouring lanes hold 16 different rows of O, which the
     // memory pipeline would write as 64 separate 8-byte pieces per instruction.  The wave
     // turns its 16 x D block around in LDS instead (the ring is free by now) and stores whole
@@ -513,6 +603,11 @@ int launch_ks(const AttnParams& p, hipStream_t stream) {
     int stages = tiles < 2 ? 2 : (tiles > kMaxStages ? kMaxStages : tiles);
     size_t lds = mfma16_lds_bytes<D, M>(p.max_anc, stages);
     while (lds > 160 * 1024 && stages > 2) lds = mfma16_lds_bytes<D, M>(p.max_anc, --stages);
+    // the kernel's start-up parks Q in the last ring slots and requests up to two leaf tiles
+    // into the first ones; ancestor lists too long to leave that much LDS go to the other kernel
+    constexpr int kWaves = M / 16 * KS, kQSlots = (kWaves * 16 + 2 * kTileN - 1) / (2 * kTileN);
+    if (stages < kQSlots + (M / 32 < 2 ? M / 32 : 2))
+        return launch_attention_mfma(p, BF16 ? FSTA_BF16 : FSTA_F16, D, BF16 && !SPLIT, stream);
     // the epilogue reuses the front of the segment: exchange area of a key split, row staging
     constexpr size_t kEpilogueBytes = KS > 1 ? (size_t)(M / 16) * (2 + D / 4) * 256 : (size_t)M * (D * 2 + 16);
     if (lds < kEpilogueBytes) lds = kEpilogueBytes;
@@ -524,7 +619,7 @@ int launch_ks(const AttnParams& p, hipStream_t stream) {
     const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
     const unsigned grid = (unsigned)(kXcds * slices_per_xcd * p.nb);
     hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT, KS>), dim3(grid), dim3(M * 4 * KS), lds, stream, p,
-                       stages);
+                       stages, grid <= kCus ? 1 : 0);
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
 }

@@ -18,6 +18,7 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kTileN = 32;     // keys per tile
+constexpr int kCus = 256;      // compute units of an MI355X
 constexpr int kXcds = 8;       // L2 domains of an MI355X; workgroup i runs on XCD i % 8
 constexpr int kMaxStages = 4;  // ring depth limit (LDS per workgroup = stages * 4 * 32 * D bytes)
 constexpr float kRescaleSlack = 8.f;  // log2 of the largest weight kept without raising the maximum
@@ -131,10 +132,32 @@ __device__ __forceinline__ u32x2 lds_read_b64(uint32_t addr) {
     asm volatile("ds_read_b64 %0, %1" : "=v"(out) : "v"(addr) : "memory");
     return out;
 }
+// 8-byte global load the compiler does not see: with global->LDS transfers in flight its own
+// wait for a loaded register is always vmcnt(0), i.e. for every transfer issued since.  The
+// result is valid after a wait_vmcnt<N>() that covers it, followed by lds_tie().
+__device__ __forceinline__ u32x2 global_read_b64(const void* ptr) {
+    u32x2 out;
+    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(out) : "v"(ptr) : "memory");
+    return out;
+}
+// LDS store the compiler does not see either (same reason); complete after lds_wait().
+__device__ __forceinline__ void lds_write_b32(uint32_t addr, uint32_t value) {
+    asm volatile("ds_write_b32 %0, %1" : : "v"(addr), "v"(value) : "memory");
+}
 // Waits for every outstanding LDS access of this wave.
 __device__ __forceinline__ void lds_wait() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 // Orders every later use of `x` behind the preceding lds_wait().
 template <typename V> __device__ __forceinline__ void lds_tie(V& x) { asm volatile("" : "+v"(x)); }
+
+// Workgroup barrier without the memory fence of __syncthreads(): that fence waits for every
+// outstanding global->LDS transfer (vmcnt(0)) and would drain the gather ring at every step.
+// What must be visible across the barrier is waited for explicitly instead: the caller's own
+// transfers of the tiles about to be used (wait_tiles_outstanding) and, here, its LDS accesses.
+__device__ __forceinline__ void ring_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
 
 struct VPair { s16x4 a, b; };   // 8 consecutive k-indices of one A-operand row
 

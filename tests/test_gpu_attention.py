@@ -204,6 +204,42 @@ def test_ancestor_slots_with_holes_and_out_of_range_ids_are_skipped():
         assert_close(o, want, torch.float32, "holes")
 
 
+@pytest.mark.parametrize("block_m,prefix,variant", [(32, 0, "default"), (64, 0, "default"), (128, 0, "default"),
+                                                    (64, 64, "default"), (64, 0, "wide"), (64, 0, "generic")])
+def test_leaf_slots_naming_other_rows(block_m, prefix, variant):
+    """A leaf slot holds a key row (reference fstattention.py:86-91 gathers K[leaf_idx]); the
+    precompute always puts the row's own id there, but the kernels must honour any id.  Leaf row
+    i is pointed at key i+1 (never one of its ancestors, parents come first) and the dense
+    oracle's mask is edited the same way."""
+    n, d, dtype = 2 * block_m, 64, torch.bfloat16
+    parent = trees.random_recursive_parents(n, 11)
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(parent, block_m)
+    mask = tp.dense_tree_mask(parent)
+    l_new = l_idx.clone()
+    for j in range(l_idx.shape[0]):
+        for r in range(block_m):
+            i = int(l_idx[j, r])
+            if i >= 0:
+                other = min(i + 1, n - 1)
+                l_new[j, r] = other
+                mask[i, i] = False
+                mask[i, other] = True
+    assert not torch.equal(l_new, l_idx)
+    q, k, v = rand_qkv(1, 2, n, n + prefix, d, dtype, 5)
+    want, _ = da_dense(q, k, v, mask, prefix, 0.125)
+    if prefix:
+        a_idx, l_new = shift_for_prefix(a_idx, l_new, prefix)
+    o = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_new.cuda(), 0.125,
+                      BLOCK_M=block_m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32,
+                      generic=variant == "generic", wide_waves=variant == "wide")
+    assert_close(o, want, dtype, f"leaf slots naming other rows, {variant}")
+
+
+def da_dense(q, k, v, tree_mask, prefix, scale):
+    from oracle import dense_attention as da
+    return da.dense_tree_attention(q, k, v, da.full_mask_with_prefix(tree_mask, prefix), scale, dtype=torch.float64)
+
+
 def test_rows_without_any_key_give_zero():
     a_idx = torch.full((1, 8), -1, dtype=torch.int64)
     a_mask = torch.zeros((1, 16, 8), dtype=torch.bool)
