@@ -446,8 +446,11 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
         float mx_raw = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
-            const bool on = (wsh >> (16 * (r / 4) + (r % 4))) & 1u;
-            sv[r] = on ? s[r / 4][r % 4] : -INFINITY;
+            // bit -> all-ones / all-zeros (v_bfe_i32), then a bitwise select against -inf (v_bfi_b32)
+            const uint32_t keep = (uint32_t)__builtin_amdgcn_sbfe((int)wsh, 16 * (r / 4) + (r % 4), 1);
+            const float score = s[r / 4][r % 4];   // (a copy: bit_cast straight from a vector element reads element 0)
+            const uint32_t bits = __builtin_bit_cast(uint32_t, score);
+            sv[r] = __builtin_bit_cast(float, (bits & keep) | (0xff800000u & ~keep));
             mx_raw = fmaxf(mx_raw, sv[r]);
         }
         mx_raw = fmaxf(mx_raw, __shfl_xor(mx_raw, 16));
