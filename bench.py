@@ -38,10 +38,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 INFINITY_CACHE_BYTES = 256 << 20
 
 # HBM bytes per launch of the headline kernel (256-node tree, cold buffers) from two
-# rocprofv3 --pmc runs, see profiles/attn_mfma_kernel_cfg2_medusa256_hbm_traffic.txt:
-# FETCH_SIZE 3202 KiB x 2.0 (a plain 256 MiB copy reads 131084 KiB on this counter, i.e. the
+# rocprofv3 --pmc runs, see profiles/attn_mfma16_kernel_cfg2_medusa256_hbm_traffic.txt:
+# FETCH_SIZE 3173.5 KiB x 2.0 (a plain 256 MiB copy reads 131084 KiB on this counter, i.e. the
 # counter sees half of the read traffic) + WRITE_SIZE 2080 KiB x 1.0 (the copy reads 262144).
-MEASURED_TRAFFIC_BYTES = (3202 * 2 + 2080) * 1024
+MEASURED_TRAFFIC_BYTES = int((3173.5 * 2 + 2080) * 1024)
 
 
 def parse_args():
@@ -325,7 +325,7 @@ def main():
         "parity": {"max_abs_err_vs_oracle": max_err, "tol": tol, "ok": ok},
         "roofline": {
             "bound": "hbm",
-            "kernel": "attn_mfma16_kernel<bf16, D=128, M=64, split P>" if args.config == 2 else "attn_mfma16_kernel",
+            "kernel": "attn_mfma16_kernel<bf16, D=128, M=64, split P, 2 key shares>" if args.config == 2 else "attn_mfma16_kernel",
             "achieved": round(achieved, 2),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
