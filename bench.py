@@ -65,13 +65,18 @@ def parse_args():
 class Workload:
     """Device-resident inputs of one configuration, in `sets` rotating copies."""
 
-    def __init__(self, index, sets_bytes, dtype=None, heads=None, batch=None):
+    def __init__(self, index, sets_bytes, dtype=None, heads=None, batch=None, order=None):
         import torch
         from fstattention_amd import _lib, create_fst_attention_kernel_inputs, trees
         from fstattention_amd.attention import _DTYPES, _packed_for
 
         self.torch = torch
         self.cfg = cfg = trees.config(index, dtype)
+        if order is not None:
+            # the same tree with its nodes (tokens) numbered depth-first (reference README.md:19-20)
+            import dataclasses
+            new_parent, _ = trees.renumber_parents(cfg.parent, trees.dfs_order(cfg.parent, order))
+            self.cfg = cfg = dataclasses.replace(cfg, parent=new_parent)
         self.lib = _lib.load()
         self._check = _lib.check
         dev = torch.device("cuda", 0)
@@ -361,6 +366,22 @@ def main():
                 "gpu_precompute_us": round(time_precompute(w) * 1e6, 2),
                 "parity_ok": ok_i, "max_abs_err": err_i,
                 "batch": w.z, "heads": w.h, "max_ancestors": w.max_anc,
+            }
+            del w
+            torch.cuda.empty_cache()
+        # the same four trees with tokens laid out depth-first: fewer K/V rows per block, so the
+        # byte count changes with the time; both are reported
+        for idx in (2, 3, 4, 5):
+            w = Workload(idx, sets_bytes=2 * INFINITY_CACHE_BYTES, order="light_first")
+            ok_i, err_i, _ = w.check_parity()
+            steps = max(20, min(args.steps, 100 if idx == 5 else args.steps))
+            ti = summarize(w, steps, min(args.warmup, 10), use_graph, False)
+            ks = ti["cold_event_us"] * 1e-6
+            extra[w.cfg.name + "_depth_first"] = {
+                "us_per_call_cold": round(ti["cold_us"], 2), "kv_rows_per_head": w.kv_rows,
+                "kv_bytes_per_call": w.kv_bytes, "kv_gbps_cold": round(w.kv_bytes / ks / 1e9, 1),
+                "hbm_frac": round(w.kv_bytes / ks / 1e9 / HBM_PEAK_GBPS, 4),
+                "parity_ok": ok_i, "max_abs_err": err_i, "max_ancestors": w.max_anc,
             }
             del w
             torch.cuda.empty_cache()

@@ -28,6 +28,8 @@ SIGNATURES = {
                                    c_int32, c_int32, c_int32, c_float, c_uint32, c_void_p]),
     "fsta_lineage_from_parents": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
                                           c_void_p]),
+    "fsta_dfs_order": (c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_void_p]),
 }
 
 _lib = None

@@ -21,6 +21,7 @@ OBJ_DIR = os.path.join(PKG_DIR, "csrc", "_obj")
 SOURCES = [
     "fsta_capi.hip",
     "fsta_precompute.hip",
+    "fsta_tree_order.hip",
     "fsta_attention_generic.hip",
     "fsta_attention_mfma.hip",
     "fsta_attention_mfma16.hip",

@@ -147,7 +147,6 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     const int dma_row = lane / kCpr, dma_slot = lane % kCpr;
     constexpr int kQDma = 16 / kRowsPerDma;
     static_assert(kQDma >= 1, "a transfer covers at most the wave's 16 rows");
-    constexpr int kQSlots = (kWaves * 16 * D + 2 * kTileElems - 1) / (2 * kTileElems);   // ring slots Q occupies
     T* qstage = ring + (size_t)stages * 2 * kTileElems - (kWaves - wave) * 16 * D;
 #pragma unroll
     for (int i = 0; i < kQDma; ++i) {
@@ -188,7 +187,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     // This shortens the start-up chain of a launch whose workgroups all run at once; a launch
     // with several rounds of workgroups hides that chain anyway and would only pay for the
     // rows of empty slots, so the launcher asks for it (`early_leaf`) for small grids only.
-    constexpr int kEarlyTiles = kLeafTiles < 2 ? kLeafTiles : 2;   // the launcher provides kQSlots + 2 ring slots
+    constexpr int kEarlyTiles = kLeafTiles < 2 ? kLeafTiles : 2;   // the launcher provides ring slots for Q plus these
     const int n_spec = early_leaf ? kEarlyTiles : 0;
 #pragma unroll
     for (int t = 0; t < kEarlyTiles; ++t) {

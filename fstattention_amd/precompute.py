@@ -117,3 +117,38 @@ def lineage_from_parents_gpu(parent: torch.Tensor, width: Optional[int] = None, 
         if st & _lib.PRE_BAD_LEVEL:
             raise ValueError(f"tree is deeper than width={width}")
     return lineage, level
+
+
+def dfs_order_gpu(parent: torch.Tensor, children: str = "index", check: bool = True):
+    """``parent [N]`` int64 on the GPU -> ``(perm, rank)`` int64 ``[N]`` on the GPU.
+
+    Device version of ``trees.dfs_order`` (``perm[new] = old``, ``rank[old] = new``) for trees
+    that are rebuilt on the GPU every decoding step; no host synchronisation with
+    ``check=False``.  ``renumber_parents_gpu`` applies the order to the tree, ``index_select``
+    to the token tensors.
+    """
+    if not parent.is_cuda or parent.dtype != torch.int64 or parent.dim() != 1:
+        raise ValueError("parent must be a 1-D int64 tensor on the GPU")
+    if children not in ("index", "light_first"):
+        raise ValueError(f"children={children!r}: expected 'index' or 'light_first'")
+    lib = _lib.load()
+    parent = parent.contiguous()
+    dev = parent.device
+    n = parent.shape[0]
+    perm = torch.empty((n,), dtype=torch.int64, device=dev)
+    rank = torch.empty((n,), dtype=torch.int64, device=dev)
+    work = torch.empty((2 * n,), dtype=torch.int32, device=dev)
+    status = torch.zeros((1,), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(lib.fsta_dfs_order(parent.data_ptr(), n, 1 if children == "light_first" else 0,
+                                      perm.data_ptr(), rank.data_ptr(), work.data_ptr(),
+                                      status.data_ptr(), _stream_ptr(dev)))
+    if check and int(status.item()) & _lib.PRE_BAD_NODE_ID:
+        raise ValueError("parent[i] must lie in [-1, i)")
+    return perm, rank
+
+
+def renumber_parents_gpu(parent: torch.Tensor, perm: torch.Tensor, rank: torch.Tensor) -> torch.Tensor:
+    """Parent array of the same forest after node ``perm[new]`` has been renamed ``new``."""
+    old_parent = parent.index_select(0, perm)
+    return torch.where(old_parent >= 0, rank.index_select(0, old_parent.clamp(min=0)), old_parent)

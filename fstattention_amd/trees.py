@@ -84,6 +84,79 @@ def parents_from_lineage(lineage, level_lookup) -> np.ndarray:
 # --------------------------------------------------------------------------- #
 # the reference's own benchmark tree
 # --------------------------------------------------------------------------- #
+# --------------------------------------------------------------------------- #
+# lineage-aware node order (the reference's open item, README.md:19-20)
+# --------------------------------------------------------------------------- #
+def subtree_sizes(parent) -> np.ndarray:
+    """Number of nodes in the subtree of every node (itself included)."""
+    parent = np.asarray(parent, dtype=np.int64)
+    size = np.ones(parent.shape[0], dtype=np.int64)
+    for i in range(parent.shape[0] - 1, 0, -1):      # children come after their parents
+        if parent[i] >= 0:
+            size[parent[i]] += size[i]
+    return size
+
+
+def dfs_order(parent, children: str = "index") -> np.ndarray:
+    """Depth-first (pre-order) numbering of a forest: ``perm[new_id] = old_id``.
+
+    Blocks of consecutive ids then hold whole subtrees and paths, so the nodes
+    of a block share most of their ancestors and the per-block ancestor lists
+    (reference ``utils.py:116-120``) shrink.  Siblings (and roots) are visited
+    by ascending id (``children="index"``) or smallest subtree first
+    (``"light_first"``, ties by id), which leaves the long paths for last and
+    packs the short ones next to their parent.  A parent still precedes its
+    children, so the result is a valid numbering for every function here.
+    """
+    parent = np.asarray(parent, dtype=np.int64)
+    n = parent.shape[0]
+    if children not in ("index", "light_first"):
+        raise ValueError(f"children={children!r}: expected 'index' or 'light_first'")
+    levels_from_parents(parent)                      # validates parent[i] < i
+    size = subtree_sizes(parent)
+    kids = [[] for _ in range(n)]
+    roots = []
+    for i in range(n):
+        (roots if parent[i] < 0 else kids[parent[i]]).append(i)
+    if children == "light_first":
+        key = lambda x: (size[x], x)
+        roots.sort(key=key)
+        for c in kids:
+            c.sort(key=key)
+    perm = np.empty(n, dtype=np.int64)
+    stack = roots[::-1]
+    filled = 0
+    while stack:
+        x = stack.pop()
+        perm[filled] = x
+        filled += 1
+        stack.extend(kids[x][::-1])
+    assert filled == n
+    return perm
+
+
+def renumber_parents(parent, perm):
+    """The same forest with node ``perm[new]`` renamed ``new``: ``(new_parent, rank)``.
+
+    ``rank[old] = new`` is the inverse of ``perm``.  Token tensors laid out in the
+    old order are brought to the new one with ``x.index_select(2, perm)`` (q, and
+    the tree part of k and v) and results back with ``o.index_select(2, rank)``.
+    ``perm`` must keep parents in front of their children.
+    """
+    parent = np.asarray(parent, dtype=np.int64)
+    perm = np.asarray(perm, dtype=np.int64)
+    n = parent.shape[0]
+    if perm.shape != (n,) or not np.array_equal(np.sort(perm), np.arange(n)):
+        raise ValueError("perm is not a permutation of the node ids")
+    rank = np.empty(n, dtype=np.int64)
+    rank[perm] = np.arange(n, dtype=np.int64)
+    old_parent = parent[perm]
+    new_parent = np.where(old_parent >= 0, rank[np.maximum(old_parent, 0)], -1)
+    if n and (new_parent >= np.arange(n)).any():
+        raise ValueError("perm puts a child in front of its parent")
+    return new_parent, rank
+
+
 def _level_starts(depth: int, topk: int, left_weight_factor: float) -> np.ndarray:
     starts = np.zeros(depth + 2, dtype=np.int64)
     size = topk

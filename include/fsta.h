@@ -133,6 +133,21 @@ int fsta_lineage_from_parents(const int64_t* parent, int64_t n_nodes, int64_t wi
                               int64_t* lineage, int64_t* level_lookup, uint32_t* status,
                               void* stream);
 
+/*
+ * Depth-first (pre-order) renumbering of a forest, the node order the reference
+ * names as its open item (README.md:19-20: blocks of consecutive ids then share
+ * lineage and their ancestor lists shrink).  parent[n_nodes] int64 as above ->
+ * perm[new_id] = old_id and rank[old_id] = new_id, both int64 [n_nodes].
+ * Siblings (and roots) are visited by ascending id, or smallest subtree first
+ * (ties by id) when light_first != 0.  workspace: 2 * n_nodes int32 of device
+ * scratch.  `status` (zero on entry) gets FSTA_PRE_BAD_NODE_ID for a parent
+ * entry outside [-1, i); perm and rank are then the identity.
+ * n_nodes <= FSTA_DFS_ORDER_MAX_NODES.
+ */
+#define FSTA_DFS_ORDER_MAX_NODES 16384
+int fsta_dfs_order(const int64_t* parent, int64_t n_nodes, int32_t light_first, int64_t* perm,
+                   int64_t* rank, int32_t* workspace, uint32_t* status, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

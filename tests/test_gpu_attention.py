@@ -10,7 +10,8 @@ import numpy as np
 import pytest
 import torch
 
-from fstattention_amd import (create_fst_attention_kernel_inputs, fst_attention, shift_for_prefix,
+from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, fst_attention,
+                              lineage_from_parents_gpu, renumber_parents_gpu, shift_for_prefix,
                               trees)
 from helpers import TOL, assert_close, dense_oracle, oracle_inputs, rand_qkv
 from oracle import tree_precompute as tp
@@ -238,6 +239,26 @@ def test_leaf_slots_naming_other_rows(block_m, prefix, variant):
 def da_dense(q, k, v, tree_mask, prefix, scale):
     from oracle import dense_attention as da
     return da.dense_tree_attention(q, k, v, da.full_mask_with_prefix(tree_mask, prefix), scale, dtype=torch.float64)
+
+
+@pytest.mark.parametrize("index,children", [(2, "index"), (2, "light_first"), (3, "index"), (5, "light_first")])
+def test_depth_first_renumbered_tree_gives_the_same_attention(index, children):
+    """Tokens laid out in depth-first order (reference README.md:19-20): the op on the renumbered
+    tree and permuted q/k/v, un-permuted, is the dense oracle's result on the tree as given."""
+    cfg = trees.config(index)
+    n, m, d = cfg.n_nodes, cfg.block_m, cfg.head_dim
+    q, k, v = rand_qkv(1, 2, n, n, d, cfg.dtype, 77)
+    scale = 1.0 / math.sqrt(d)
+    want, _ = dense_oracle(q, k, v, cfg.parent, scale)
+    perm, rank = dfs_order_gpu(torch.from_numpy(cfg.parent).cuda(), children)
+    new_parent = renumber_parents_gpu(torch.from_numpy(cfg.parent).cuda(), perm, rank)
+    lineage, level = lineage_from_parents_gpu(new_parent)
+    max_anc = trees.required_max_ancestors(new_parent.cpu().numpy(), m)
+    a_idx, a_mask, l_idx = create_fst_attention_kernel_inputs(lineage, level, m, max_anc)
+    qp, kp, vp = (t.cuda().index_select(2, perm) for t in (q, k, v))
+    o = fst_attention(qp, kp, vp, a_idx, a_mask, l_idx, scale, BLOCK_M=m, MAX_ANCESTORS=max_anc,
+                      out_dtype=torch.float32)
+    assert_close(o.index_select(2, rank), want, cfg.dtype, f"{cfg.name} in depth-first order")
 
 
 def test_rows_without_any_key_give_zero():

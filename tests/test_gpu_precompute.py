@@ -4,8 +4,8 @@ import pytest
 import torch
 
 from conftest import golden_cases
-from fstattention_amd import (create_fst_attention_kernel_inputs, lineage_from_parents_gpu,
-                              pack_tree_mask, trees)
+from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, lineage_from_parents_gpu,
+                              pack_tree_mask, renumber_parents_gpu, trees)
 from oracle import tree_precompute as tp
 
 pytestmark = pytest.mark.gpu
@@ -144,3 +144,34 @@ def test_lineage_from_parents_on_gpu():
         lineage_from_parents_gpu(torch.tensor([-1, 0, 5], dtype=torch.int64).cuda())
     with pytest.raises(ValueError):
         lineage_from_parents_gpu(torch.tensor([-1, 0, 1, 2], dtype=torch.int64).cuda(), width=2)
+
+
+@pytest.mark.parametrize("children", ["index", "light_first"])
+def test_dfs_order_on_gpu_matches_the_host_order(children):
+    cases = [np.array([-1], dtype=np.int64), np.array([-1, -1, -1], dtype=np.int64)]
+    for seed, n, window in [(1, 2, None), (2, 300, None), (3, 1500, 8), (4, 2049, 64)]:
+        parent = trees.random_recursive_parents(n, seed, window)
+        parent[::101] = -1                      # forest
+        cases.append(parent)
+    cases += [trees.config(i).parent for i in (2, 3, 4, 5)]
+    for parent in cases:
+        want = trees.dfs_order(parent, children)
+        dev_parent = torch.from_numpy(parent).cuda()
+        perm, rank = dfs_order_gpu(dev_parent, children)
+        np.testing.assert_array_equal(perm.cpu().numpy(), want)
+        want_parent, want_rank = trees.renumber_parents(parent, want)
+        np.testing.assert_array_equal(rank.cpu().numpy(), want_rank)
+        np.testing.assert_array_equal(renumber_parents_gpu(dev_parent, perm, rank).cpu().numpy(), want_parent)
+
+
+def test_dfs_order_on_gpu_flags_bad_parents_and_sizes():
+    with pytest.raises(ValueError):
+        dfs_order_gpu(torch.tensor([-1, 0, 5, 1], dtype=torch.int64).cuda())
+    with pytest.raises(ValueError):
+        dfs_order_gpu(torch.tensor([-1, 1, 0], dtype=torch.int64).cuda())
+    perm, rank = dfs_order_gpu(torch.tensor([-1, -3, 0], dtype=torch.int64).cuda(), check=False)
+    assert perm.tolist() == [0, 1, 2] and rank.tolist() == [0, 1, 2]   # identity when flagged
+    with pytest.raises(RuntimeError):
+        dfs_order_gpu(torch.full((16385,), -1, dtype=torch.int64).cuda())
+    empty, _ = dfs_order_gpu(torch.empty((0,), dtype=torch.int64).cuda())
+    assert empty.numel() == 0

@@ -5,6 +5,7 @@ import torch
 
 from conftest import golden_cases
 from fstattention_amd import trees
+from oracle import tree_precompute as tp
 
 
 @pytest.mark.parametrize("case", [c for c in golden_cases() if c.startswith("create_tree")])
@@ -100,3 +101,79 @@ def test_make_qkv_is_seeded_on_cpu():
     assert torch.equal(q1, q2)
     q3, k3, _ = trees.make_qkv(cfg, prefix=32)
     assert k3.shape[2] == 96
+
+
+# --------------------------------------------------------------------------- #
+# depth-first renumbering (the reference's open item, README.md:19-20)
+# --------------------------------------------------------------------------- #
+def _recursive_preorder(parent, light_first):
+    """Textbook recursive pre-order, children in the stated order."""
+    n = len(parent)
+    kids = {i: [] for i in range(-1, n)}
+    for i, p in enumerate(parent):
+        kids[int(p)].append(i)
+
+    def size(x):
+        return 1 + sum(size(c) for c in kids[x])
+
+    out = []
+
+    def visit(x):
+        if x >= 0:
+            out.append(x)
+        order = sorted(kids[x], key=(lambda c: (size(c), c)) if light_first else (lambda c: c))
+        for c in order:
+            visit(c)
+
+    visit(-1)
+    return np.asarray(out, dtype=np.int64)
+
+
+@pytest.mark.parametrize("children", ["index", "light_first"])
+def test_dfs_order_is_the_textbook_preorder(children):
+    rng = np.random.default_rng(3)
+    for n in (1, 2, 7, 33, 150):
+        for _ in range(4):
+            parent = np.array([-1] + [int(rng.integers(-1, i)) for i in range(1, n)], dtype=np.int64)  # forests too
+            perm = trees.dfs_order(parent, children)
+            np.testing.assert_array_equal(perm, _recursive_preorder(parent, children == "light_first"))
+
+
+def test_renumbered_tree_is_the_same_tree():
+    parent = trees.random_recursive_parents(200, 9)
+    perm = trees.dfs_order(parent)
+    new_parent, rank = trees.renumber_parents(parent, perm)
+    np.testing.assert_array_equal(rank[perm], np.arange(200))
+    assert (new_parent < np.arange(200)).all()                 # still a topological numbering
+    old_mask = tp.dense_tree_mask(parent)
+    new_mask = tp.dense_tree_mask(new_parent)
+    np.testing.assert_array_equal(new_mask, old_mask[np.ix_(perm, perm)])
+    # a depth-first numbered tree is a fixed point
+    np.testing.assert_array_equal(trees.dfs_order(new_parent), np.arange(200))
+    # in pre-order every subtree is a run of consecutive ids
+    size = trees.subtree_sizes(new_parent)
+    for i in range(200):
+        assert new_mask[i + 1:i + size[i], i].all() and not new_mask[i + size[i]:, i].any()
+
+
+def test_dfs_order_shrinks_the_ancestor_lists_of_the_benchmark_trees():
+    for index, at_most in ((2, 0.75), (5, 0.60)):
+        cfg = trees.config(index)
+        rows = {}
+        for name, parent in (("given", cfg.parent),
+                             ("dfs", trees.renumber_parents(cfg.parent, trees.dfs_order(cfg.parent))[0])):
+            lineage, level = trees.lineage_from_parents(parent)
+            max_anc = trees.required_max_ancestors(parent, cfg.block_m)
+            a_idx, _, l_idx = tp.block_inputs(lineage.numpy().copy(), level.numpy(), cfg.block_m, max_anc)
+            rows[name] = tp.kv_rows_loaded(a_idx, l_idx)
+        assert rows["dfs"] <= at_most * rows["given"], rows
+
+
+def test_renumber_rejects_bad_orders():
+    parent = np.array([-1, 0, 1, 1], dtype=np.int64)
+    with pytest.raises(ValueError):
+        trees.renumber_parents(parent, np.array([0, 1, 1, 3]))
+    with pytest.raises(ValueError):
+        trees.renumber_parents(parent, np.array([1, 0, 2, 3]))   # child before parent
+    with pytest.raises(ValueError):
+        trees.dfs_order(parent, children="random")
