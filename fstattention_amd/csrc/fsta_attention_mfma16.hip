@@ -69,6 +69,9 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     constexpr int kSteps = D / 32;                // MFMAs per 16-key half of S^T
     constexpr int kDTiles = D / 16;               // 16-row tiles of O^T
     constexpr int kTileElems = kTileN * D;
+    // Largest sum of a lane's 8 weights accepted without looking at the row maximum: far from
+    // float overflow in l and O, and every single weight still converts to the 16-bit type.
+    constexpr float kTrustedSum = BF16 ? 16777216.f : 32768.f;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     T* ring = reinterpret_cast<T*>(smem);                 // [stages][K tile | V tile]
@@ -437,12 +440,10 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
         };
         VPair v0[kHalf], v1[kHalf];
         read_v(v0, 0);
-        // mask + online softmax; register j of half `sub` is key 16*sub + 4g + j.  The maximum is
-        // taken over the raw scores (the scale is positive here) and the scale rides in the FMA
-        // under the exp2.
+        // mask + online softmax; register j of half `sub` is key 16*sub + 4g + j.  The scale rides
+        // in the FMA under the exp2.
         const uint32_t wsh = word >> (4 * g);
         float sv[8];
-        float mx_raw = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
             // bit -> all-ones / all-zeros (v_bfe_i32), then a bitwise select against -inf (v_bfi_b32)
@@ -450,15 +451,31 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
             const float score = s[r / 4][r % 4];   // (a copy: bit_cast straight from a vector element reads element 0)
             const uint32_t bits = __builtin_bit_cast(uint32_t, score);
             sv[r] = __builtin_bit_cast(float, (bits & keep) | (0xff800000u & ~keep));
-            mx_raw = fmaxf(mx_raw, sv[r]);
         }
-        mx_raw = fmaxf(mx_raw, __shfl_xor(mx_raw, 16));
-        mx_raw = fmaxf(mx_raw, __shfl_xor(mx_raw, 32));
-        const float mx = mx_raw * p.scale_log2e;
-        // Raise the running maximum only for rows that would otherwise produce a weight above
-        // 2^kRescaleSlack (always when the row had no key so far): a rare wave-uniform branch.
-        const bool raise = mx > m_i + kRescaleSlack || (m_i == -INFINITY && mx > -INFINITY);
-        if (__ballot(raise) != 0ull) {
+        // The weights are first taken against the running maximum as it stands: no row maximum,
+        // no cross-lane exchange.  That is exact as long as no weight gets large (a power-of-two
+        // factor on a row's weights cancels in O / l); the sum of the lane's weights is the check.
+        // A row without a maximum so far, or a sum above the limit (or not a number), sends the
+        // wave through the full update below: row maximum, raise, rescale, weights again.
+        float pw[8];
+        float rowsum = 0.f;
+        {
+            const float neg_m = m_i == -INFINITY ? 0.f : -m_i;
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                pw[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[r], p.scale_log2e, neg_m));
+                rowsum += pw[r];
+            }
+        }
+        const bool redo = !(rowsum <= kTrustedSum) || (m_i == -INFINITY && (wsh & 0x000f000fu) != 0u);
+        if (__ballot(redo) != 0ull) {
+            float mx_raw = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
+                                 fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+            mx_raw = fmaxf(mx_raw, __shfl_xor(mx_raw, 16));
+            mx_raw = fmaxf(mx_raw, __shfl_xor(mx_raw, 32));
+            const float mx = mx_raw * p.scale_log2e;   // the scale is positive here
+            // raise only rows that would otherwise keep a weight above 2^kRescaleSlack
+            const bool raise = mx > m_i + kRescaleSlack || (m_i == -INFINITY && mx > -INFINITY);
             const float alpha = raise ? __builtin_amdgcn_exp2f(m_i - mx) : 1.f;   // exp2(-inf) = 0
             if (raise) m_i = mx;
             l_i *= alpha;
@@ -466,20 +483,20 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
             for (int dt = 0; dt < kDTiles; ++dt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
-        }
-        const float neg_m = m_i == -INFINITY ? 0.f : -m_i;
-        float rowsum = 0.f;
+            const float neg_m = m_i == -INFINITY ? 0.f : -m_i;
+            rowsum = 0.f;
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
-            sv[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[r], p.scale_log2e, neg_m));
-            rowsum += sv[r];
+            for (int r = 0; r < 8; ++r) {
+                pw[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[r], p.scale_log2e, neg_m));
+                rowsum += pw[r];
+            }
         }
         l_i += rowsum;
         // P^T fragment: the 8 weights are this lane's 8 k-slots
         u32x4 hi4, lo4;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const float a = sv[2 * e], b = sv[2 * e + 1];
+            const float a = pw[2 * e], b = pw[2 * e + 1];
             const uint32_t hi = MM::pack(a, b);
             hi4[e] = hi;
             if (SPLIT) lo4[e] = MM::pack(a - MM::low(hi), b - MM::high(hi));
