@@ -210,6 +210,12 @@ __global__ __launch_bounds__(M * 2 * key_split_for(M), 2) void attn_mfma_kernel(
         }
     };
     auto begin_step = [&](int g) {
+        if (issued < min(consumed + g, total_tiles)) {
+            // ring too shallow (long ancestor lists leave little LDS) for this step's tiles to be
+            // in flight already: free the slots first, then request them
+            ring_barrier();
+            refill();
+        }
         wait_tiles_outstanding<kDmaPerWave>(max(issued - consumed - g, 0));
         ring_barrier();
         refill();

@@ -292,6 +292,12 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
         }
     };
     auto begin_step = [&](int n) {
+        if (issued < min(consumed + n, total_tiles)) {
+            // ring too shallow (long ancestor lists leave little LDS) for this step's tiles to be
+            // in flight already: free the slots first, then request them
+            ring_barrier();
+            refill();
+        }
         wait_tiles_outstanding<kDmaPerWave>(max(issued - consumed - n, 0));
         ring_barrier();
         refill();

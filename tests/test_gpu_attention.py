@@ -261,6 +261,20 @@ def test_depth_first_renumbered_tree_gives_the_same_attention(index, children):
     assert_close(o.index_select(2, rank), want, cfg.dtype, f"{cfg.name} in depth-first order")
 
 
+def test_very_long_ancestor_lists_take_the_kernel_with_the_smaller_lds_footprint():
+    """A 4992-node chain: the last block of 128 rows has 4991 ancestors, more than the default
+    kernel can keep beside its four-stage ring; the launch must still give the right answer."""
+    n, m, d = 4992, 128, 128
+    parent = np.arange(-1, n - 1, dtype=np.int64)
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(parent, m)
+    assert max_anc >= 4991
+    q, k, v = rand_qkv(1, 1, n, n, d, torch.bfloat16, 3)
+    want, _ = dense_oracle(q, k, v, parent, 0.05)
+    o = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(), 0.05,
+                      BLOCK_M=m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32)
+    assert_close(o, want, torch.bfloat16, "4992-node chain")
+
+
 def test_rows_without_any_key_give_zero():
     a_idx = torch.full((1, 8), -1, dtype=torch.int64)
     a_mask = torch.zeros((1, 16, 8), dtype=torch.bool)
