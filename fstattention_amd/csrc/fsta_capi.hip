@@ -70,8 +70,11 @@ extern "C" int fsta_attention_fwd(const void* q, const void* k, const void* v, v
     // the matrix-core kernel takes row maxima before scaling, which needs a positive scale
     if (!(flags & FSTA_FLAG_GENERIC) && sm_scale > 0.f && mfma_supported(dtype, head_dim, block_m)) {
         const bool fast_pv = (flags & FSTA_FLAG_FAST_PV) != 0;
-        if (flags & FSTA_FLAG_WIDE_WAVES) return launch_attention_mfma(p, dtype, head_dim, fast_pv, s);
-        return launch_attention_mfma16(p, dtype, head_dim, fast_pv, s);
+        const int rc = (flags & FSTA_FLAG_WIDE_WAVES) ? launch_attention_mfma(p, dtype, head_dim, fast_pv, s)
+                                                      : launch_attention_mfma16(p, dtype, head_dim, fast_pv, s);
+        // ancestor lists too long for the LDS-resident lists of these kernels: the scalar kernel
+        // streams them and takes any length
+        if (rc != FSTA_EUNSUPPORTED) return rc;
     }
     return launch_attention_generic(p, dtype, head_dim, s);
 }

@@ -273,6 +273,15 @@ def test_very_long_ancestor_lists_take_the_kernel_with_the_smaller_lds_footprint
     o = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(), 0.05,
                       BLOCK_M=m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32)
     assert_close(o, want, torch.bfloat16, "4992-node chain")
+    # and a list no matrix-core kernel has the LDS for (falls through to the scalar kernel)
+    n = 8192
+    parent = np.arange(-1, n - 1, dtype=np.int64)
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(parent, m)
+    q, k, v = rand_qkv(1, 1, n, n, d, torch.bfloat16, 4)
+    want, _ = dense_oracle(q, k, v, parent, 0.05)
+    o = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(), 0.05,
+                      BLOCK_M=m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32)
+    assert_close(o, want, torch.bfloat16, "8192-node chain")
 
 
 def test_rows_without_any_key_give_zero():
