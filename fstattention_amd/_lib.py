@@ -30,6 +30,8 @@ SIGNATURES = {
                                           c_void_p]),
     "fsta_dfs_order": (c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_void_p]),
+    "fsta_merge_states": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
+                                  c_int32, c_int32, c_void_p]),
 }
 
 _lib = None

@@ -165,3 +165,36 @@ def shift_for_prefix(ancestor_idx: torch.Tensor, leaf_idx: torch.Tensor, prefix:
     """
     return (torch.where(ancestor_idx >= 0, ancestor_idx + prefix, ancestor_idx),
             torch.where(leaf_idx >= 0, leaf_idx + prefix, leaf_idx))
+
+
+def merge_attention_states(o_a: torch.Tensor, lse_a: torch.Tensor, o_b: torch.Tensor, lse_b: torch.Tensor):
+    """Joins two partial attention results of the same queries over disjoint key sets.
+
+    ``o_*`` ``[..., Nq, D]`` (same dtype and shape), ``lse_*`` float32 with one entry per row
+    of ``o_*`` in the same order: the base-2 log-sum-exp that ``fst_attention(...,
+    return_lse=True)`` returns (reference ``fstattention.py:139-141``).  Returns ``(o, lse)``
+    of the attention over the union of the key sets.  Typical use: the tree part from
+    ``fst_attention`` with ``Nk == Nq`` and the dense shared prefix (reference
+    ``fstattention.py:113-136``) from a kernel that reads a paged KV cache.
+    """
+    if o_a.shape != o_b.shape or o_a.dtype != o_b.dtype or o_a.dtype not in _DTYPES:
+        raise ValueError("o_a and o_b must have the same shape and a dtype of float32/float16/bfloat16")
+    if not (o_a.is_cuda and o_b.is_cuda and lse_a.is_cuda and lse_b.is_cuda):
+        raise ValueError("merge_attention_states runs on the GPU only")
+    d = o_a.shape[-1]
+    rows = o_a.numel() // d if d else 0
+    if lse_a.numel() != rows or lse_b.numel() != rows:
+        raise ValueError(f"lse tensors need one entry per row ({rows}), got {lse_a.numel()} and {lse_b.numel()}")
+    if lse_a.dtype != torch.float32 or lse_b.dtype != torch.float32:
+        raise ValueError("lse tensors must be float32")
+    if d % 8:
+        raise ValueError(f"head dim {d} is not a multiple of 8")
+    lib = _lib.load()
+    o_a, o_b, lse_a, lse_b = o_a.contiguous(), o_b.contiguous(), lse_a.contiguous(), lse_b.contiguous()
+    o = torch.empty_like(o_a)
+    lse = torch.empty_like(lse_a)
+    with torch.cuda.device(o_a.device):
+        _lib.check(lib.fsta_merge_states(o_a.data_ptr(), lse_a.data_ptr(), o_b.data_ptr(), lse_b.data_ptr(),
+                                         o.data_ptr(), lse.data_ptr(), rows, d, _DTYPES[o_a.dtype],
+                                         _stream_ptr(o_a.device)))
+    return o, lse

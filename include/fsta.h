@@ -148,6 +148,20 @@ int fsta_lineage_from_parents(const int64_t* parent, int64_t n_nodes, int64_t wi
 int fsta_dfs_order(const int64_t* parent, int64_t n_nodes, int32_t light_first, int64_t* perm,
                    int64_t* rank, int32_t* workspace, uint32_t* status, void* stream);
 
+/*
+ * Joins two partial attention results of the same queries over disjoint key
+ * sets: o = (o_a 2^lse_a + o_b 2^lse_b) / (2^lse_a + 2^lse_b) per row, lse_out
+ * (may be NULL) = log2 of the denominator.  o_*: [rows, head_dim] of `dtype`,
+ * lse_*: float32 [rows], base 2 as written by fsta_attention_fwd (reference
+ * fstattention.py:139-141, which computes L and drops it).  A part with
+ * lse = -inf carries no keys and is ignored.  With it the dense shared prefix
+ * of fstattention.py:113-136 can come from any kernel that reports its
+ * log-sum-exp.  o_out may alias o_a or o_b.  head_dim a multiple of 8.
+ */
+int fsta_merge_states(const void* o_a, const float* lse_a, const void* o_b, const float* lse_b,
+                      void* o_out, float* lse_out, int64_t rows, int32_t head_dim, int32_t dtype,
+                      void* stream);
+
 #ifdef __cplusplus
 }
 #endif

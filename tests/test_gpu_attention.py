@@ -11,7 +11,7 @@ import pytest
 import torch
 
 from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, fst_attention,
-                              lineage_from_parents_gpu, renumber_parents_gpu, shift_for_prefix,
+                              lineage_from_parents_gpu, merge_attention_states, renumber_parents_gpu, shift_for_prefix,
                               trees)
 from helpers import TOL, assert_close, dense_oracle, oracle_inputs, rand_qkv
 from oracle import tree_precompute as tp
@@ -282,6 +282,42 @@ def test_very_long_ancestor_lists_take_the_kernel_with_the_smaller_lds_footprint
     o = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(), 0.05,
                       BLOCK_M=m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32)
     assert_close(o, want, torch.bfloat16, "8192-node chain")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_prefix_and_tree_parts_merge_into_the_full_result(dtype):
+    """Attention over [prefix | tree] = the two parts computed apart and joined through their
+    log-sum-exp (what exposing L of reference fstattention.py:139-141 is for).  Checked against
+    the dense oracle over all keys, so the merge formula is pinned by the identity, not retyped."""
+    parent = trees.random_recursive_parents(128, 21)
+    m, d, prefix, scale = 64, 64, 96, 0.2
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(parent, m)
+    q, k, v = rand_qkv(2, 2, 128, 128 + prefix, d, dtype, 8)
+    want, want_lse = dense_oracle(q, k, v, parent, scale, prefix=prefix)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    kw = dict(BLOCK_M=m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32, return_lse=True)
+    # tree part: keys of the tree only
+    o_t, l_t = fst_attention(qd, kd[:, :, prefix:].contiguous(), vd[:, :, prefix:].contiguous(),
+                             a_idx.cuda(), a_mask.cuda(), l_idx.cuda(), scale, **kw)
+    # prefix part: same call layout, tree keys switched off (empty mask, no leaf slots)
+    o_p, l_p = fst_attention(qd, kd, vd, torch.full_like(a_idx, -1).cuda(), torch.zeros_like(a_mask).cuda(),
+                             torch.full_like(l_idx, -1).cuda(), scale, **kw)
+    o, lse = merge_attention_states(o_t, l_t, o_p, l_p)
+    assert_close(o, want, dtype, "merged")
+    tol = 1e-4 if dtype == torch.float32 else 2e-3
+    torch.testing.assert_close(lse.cpu().double().view(2, 2, 128), want_lse, atol=tol, rtol=tol)
+    # storage-type states (what a caller usually holds), an empty part, and both parts empty
+    o16, lse16 = merge_attention_states(o_t.to(dtype), l_t, o_p.to(dtype), l_p)
+    assert o16.dtype == dtype
+    torch.testing.assert_close(o16.float().cpu().double(), want, atol=1e-2 if dtype != torch.float32 else 1e-5, rtol=1e-2)
+    none = torch.full_like(l_t, float("-inf"))
+    junk = torch.full_like(o_t, float("nan"))
+    o_same, l_same = merge_attention_states(o_t, l_t, junk, none)
+    assert torch.equal(o_same, o_t) and torch.equal(l_same, l_t)
+    o_zero, l_zero = merge_attention_states(junk, none, junk, none)
+    assert (o_zero == 0).all() and torch.isinf(l_zero).all() and (l_zero < 0).all()
+    with pytest.raises(ValueError):
+        merge_attention_states(o_t, l_t[:, :5], o_p, l_p)
 
 
 def test_rows_without_any_key_give_zero():
