@@ -150,7 +150,11 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     const int dma_row = lane / kCpr, dma_slot = lane % kCpr;
     constexpr int kQDma = 16 / kRowsPerDma;
     static_assert(kQDma >= 1, "a transfer covers at most the wave's 16 rows");
-    T* qstage = ring + (size_t)stages * 2 * kTileElems - (kWaves - wave) * 16 * D;
+    // (a small grid has LDS to spare: Q then gets an area of its own behind the mask words, the
+    // whole ring is free from the start and the fragments are read after the ancestor tiles have
+    // been requested instead of in front of the first barrier)
+    T* qstage = early_leaf ? reinterpret_cast<T*>(mask_s + anc_tile_capacity(p.max_anc) * M) + wave * 16 * D
+                           : ring + (size_t)stages * 2 * kTileElems - (kWaves - wave) * 16 * D;
 #pragma unroll
     for (int i = 0; i < kQDma; ++i) {
         const int r = i * kRowsPerDma + dma_row;
@@ -247,9 +251,9 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     }
     // Q fragments: B operand of S^T = K.Q^T, lane holds Q[q][32s + 8g .. +7].  Only the leaf
     // tiles requested above were issued after the Q rows.
-    wait_tiles_outstanding<kDmaPerWave>(gathers ? n_spec : 0);
     Frag qf[kSteps];
-    {
+    auto read_q = [&](int tiles_issued_since) {
+        wait_tiles_outstanding<kDmaPerWave>(gathers ? tiles_issued_since : 0);
         u32x4 qraw[kSteps];
 #pragma unroll
         for (int s = 0; s < kSteps; ++s)
@@ -260,7 +264,8 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
             lds_tie(qraw[s]);
             qf[s] = __builtin_bit_cast(Frag, qraw[s]);
         }
-    }
+    };
+    if (!early_leaf) read_q(0);   // Q sits in ring slots the gathers are about to take
     n_anc = min(max(n_anc, 0), p.max_anc);
     const int listed_tiles = kLeafTiles + (n_anc + kTileN - 1) / kTileN;
     const int total_tiles = listed_tiles + (p.prefix + kTileN - 1) / kTileN;
@@ -325,6 +330,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
         }
     }
     refill();
+    if (early_leaf) read_q(issued);
 
     float m_i = -INFINITY, l_i = 0.f;
     f32x4 o[kDTiles];
@@ -638,13 +644,17 @@ int launch_ks(const AttnParams& p, hipStream_t stream) {
     if (lds < kEpilogueBytes) lds = kEpilogueBytes;
     if (lds > 160 * 1024)
         return fail(FSTA_EUNSUPPORTED, "max_ancestors=%d needs %zu bytes of LDS (limit 163840)", p.max_anc, lds);
+    const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
+    const unsigned grid = (unsigned)(kXcds * slices_per_xcd * p.nb);
+    // a launch whose workgroups all run at once: leaf tiles requested early, Q in an area of its own
+    constexpr size_t kQBytes = (size_t)kWaves * 16 * D * 2;
+    const int early = grid <= kCus && lds + kQBytes <= 160 * 1024 ? 1 : 0;
+    if (early) lds += kQBytes;
     if (lds > 64 * 1024)
         FSTA_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_mfma16_kernel<BF16, D, M, SPLIT, KS>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
-    const unsigned grid = (unsigned)(kXcds * slices_per_xcd * p.nb);
     hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT, KS>), dim3(grid), dim3(M * 4 * KS), lds, stream, p,
-                       stages, grid <= kCus ? 1 : 0);
+                       stages, early);
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
 }
