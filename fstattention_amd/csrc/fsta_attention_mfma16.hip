@@ -348,11 +348,15 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
             const T* vt = kt + kTileElems;
             const int row = (qgroup & 1) * 16 + ql;   // this query's row of the leaf tile
             float part[2] = {0.f, 0.f};
+            u32x2 vraw[kDTiles];   // the row's V values are requested together with its K values
             {
                 u32x4 kraw[kSteps];
 #pragma unroll
                 for (int ks = 0; ks < kSteps; ++ks)
                     kraw[ks] = lds_read_b128(lds_addr(kt + row * D + k_chunk<D>(row, 4 * ks + g) * 8));
+#pragma unroll
+                for (int dt = 0; dt < kDTiles; ++dt)   // accumulator rows 4g .. 4g+3 of tile dt: 4 head dims
+                    vraw[dt] = lds_read_b64(lds_addr(vt + row * D + k_chunk<D>(row, 2 * dt + (g >> 1)) * 8 + 4 * (g & 1)));
                 lds_wait();
 #pragma unroll
                 for (int ks = 0; ks < kSteps; ++ks) {
@@ -366,14 +370,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
                     }
                 }
             }
-            float dot = part[0] + part[1];
-            dot += __shfl_xor(dot, 16);
-            dot += __shfl_xor(dot, 32);
-            u32x2 vraw[kDTiles];
-#pragma unroll
-            for (int dt = 0; dt < kDTiles; ++dt)   // accumulator rows 4g .. 4g+3 of tile dt: 4 head dims
-                vraw[dt] = lds_read_b64(lds_addr(vt + row * D + k_chunk<D>(row, 2 * dt + (g >> 1)) * 8 + 4 * (g & 1)));
-            lds_wait();
+            const float dot = sum_quarters(part[0] + part[1]);
 #pragma unroll
             for (int dt = 0; dt < kDTiles; ++dt) lds_tie(vraw[dt]);
             if (leaf_ok) {
@@ -483,8 +480,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
         if (__ballot(redo) != 0ull) {
             float mx_raw = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
                                  fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-            mx_raw = fmaxf(mx_raw, __shfl_xor(mx_raw, 16));
-            mx_raw = fmaxf(mx_raw, __shfl_xor(mx_raw, 32));
+            mx_raw = max_quarters(mx_raw);
             const float mx = mx_raw * p.scale_log2e;   // the scale is positive here
             // raise only rows that would otherwise keep a weight above 2^kRescaleSlack
             const bool raise = mx > m_i + kRescaleSlack || (m_i == -INFINITY && mx > -INFINITY);
@@ -563,8 +559,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     }
 
     // ---- epilogue: normalise, write O once (and the base-2 log-sum-exp) --------
-    float l_tot = l_i + __shfl_xor(l_i, 16);
-    l_tot += __shfl_xor(l_tot, 32);
+    const float l_tot = sum_quarters(l_i);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     {
         // the row number is derived again from an opaque copy: kept from the start-up it would

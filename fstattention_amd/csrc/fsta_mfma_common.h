@@ -159,6 +159,34 @@ __device__ __forceinline__ void ring_barrier() {
     asm volatile("" ::: "memory");
 }
 
+// Sum / maximum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (one per quarter-wave), result in
+// all four: v_permlane32_swap exchanges the upper half of one register with the lower half of
+// another, v_permlane16_swap the odd 16-lane rows with the even ones, so two copies of x turn
+// into "my half's value" and "the other half's value".  Vector ALU only, no trip through LDS
+// (ds_bpermute).  All 64 lanes must be active.
+__device__ __forceinline__ void swap_halves(float x, bool rows16, float& mine, float& other) {
+    const uint32_t bits = __builtin_bit_cast(uint32_t, x);
+    const u32x2 r = rows16 ? __builtin_amdgcn_permlane16_swap(bits, bits, false, false)
+                           : __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+    const uint32_t r0 = r[0], r1 = r[1];   // (copies: bit_cast straight from a vector element reads element 0)
+    mine = __builtin_bit_cast(float, r0);
+    other = __builtin_bit_cast(float, r1);
+}
+__device__ __forceinline__ float sum_quarters(float x) {
+    float a, b;
+    swap_halves(x, false, a, b);
+    x = a + b;
+    swap_halves(x, true, a, b);
+    return a + b;
+}
+__device__ __forceinline__ float max_quarters(float x) {
+    float a, b;
+    swap_halves(x, false, a, b);
+    x = fmaxf(a, b);
+    swap_halves(x, true, a, b);
+    return fmaxf(a, b);
+}
+
 struct VPair { s16x4 a, b; };   // 8 consecutive k-indices of one A-operand row
 
 // 16-byte chunk position of (row, chunk) inside an LDS tile.  K is read as whole
