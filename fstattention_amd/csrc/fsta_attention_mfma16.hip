@@ -217,9 +217,13 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
             if (c < cap * kTileN) {
                 const bool ok = ids[i] >= 0 && ids[i] < p.nk;
                 const uint64_t vote = __ballot(ok);
-                const uint32_t mine = (uint32_t)(vote >> (lane & 32));
-                const int first = mine ? (lane & 32) + __ffs(mine) - 1 : lane;
-                const int fallback = __shfl(ok ? (int)ids[i] : 0, first);
+                const uint32_t lo = (uint32_t)vote, hi = (uint32_t)(vote >> 32);   // two tiles per wave
+                const int mine_id = ok ? (int)ids[i] : 0;
+                // first valid row of each tile: wave-uniform lane numbers, so plain lane reads
+                const int first_lo = lo ? __builtin_amdgcn_readlane(mine_id, __ffs(lo) - 1) : 0;
+                const int first_hi = hi ? __builtin_amdgcn_readlane(mine_id, 31 + __ffs(hi)) : 0;
+                const uint32_t mine = lane < 32 ? lo : hi;
+                const int fallback = lane < 32 ? first_lo : first_hi;
                 lds_write_b32(lds_addr(key_s + c), ok ? (int)ids[i] : fallback);
                 if ((lane & 31) == 0) lds_write_b32(lds_addr(valid_s + (c >> 5)), mine);
             }
