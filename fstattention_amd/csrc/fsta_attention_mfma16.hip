@@ -45,6 +45,25 @@ __host__ __device__ constexpr size_t mfma16_lds_bytes(int max_anc, int stages) {
            (size_t)anc_tile_capacity(max_anc) * M * 4;
 }
 
+// 16 staged rows of W bytes each (LDS, `stride` apart) -> global rows `pitch` apart, 16 bytes per
+// lane, whole rows per instruction; rows at or past rows_valid are not written.
+template <int W>
+__device__ __forceinline__ void flush_rows(const unsigned char* stage, int stride, unsigned char* dst, size_t pitch,
+                                           int lane, int rows_valid) {
+    constexpr int kLanesPerRow = W / 16;
+    constexpr int kRowsPerStore = 64 / kLanesPerRow;
+    constexpr int kIters = kRowsPerStore >= 16 ? 1 : 16 / kRowsPerStore;
+    const int st_row = lane / kLanesPerRow, st_piece = lane % kLanesPerRow;
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) {
+        const int r = i * kRowsPerStore + st_row;
+        if (r < 16 && r < rows_valid) {
+            const u32x4 val = *reinterpret_cast<const u32x4*>(stage + r * stride + st_piece * 16);
+            *reinterpret_cast<u32x4*>(dst + r * pitch + st_piece * 16) = val;
+        }
+    }
+}
+
 // KS = waves that share one group of 16 query rows, each taking every KS-th tile with its own
 // running softmax (merged through LDS at the end).
 template <bool BF16, int D, int M, bool SPLIT, int KS>
@@ -534,21 +553,88 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
         }
     }
 
-    // ---- merge the shares of a query group (same lanes, same layout) through LDS ----
-    if (kSplit > 1) {
+    // ---- end of the tile list: normalise, write O once (and the base-2 log-sum-exp) --------
+    // In the accumulator layout 16 neighbouring lanes hold 16 different rows of O, which the
+    // memory pipeline would write as 64 separate 8-byte pieces per instruction.  A wave turns
+    // its block around in LDS instead (the ring is free by now) and stores whole rows, 16 bytes
+    // per lane; columns go in passes of at most 2*D bytes per row.
+    constexpr int kStageStride = D * 2 + 16;     // bytes per staged row (padded against bank conflicts)
+    const int first_row = j * M + qgroup * 16;
+    auto finish = [&](auto& vals, int col0, unsigned char* stage, bool write_lse) {
+        constexpr int kTilesHere = (int)(sizeof(vals) / sizeof(vals[0]));
+        const float l_tot = sum_quarters(l_i);
+        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+        if (write_lse) {
+            // the row number is derived again from an opaque copy: kept from the start-up it
+            // would occupy a register pair through the whole kernel
+            int rib = row_in_block;
+            asm volatile("" : "+v"(rib));
+            const int row = j * M + rib;
+            if (row < p.nq && p.lse && g == 0)
+                p.lse[(size_t)hz * p.nq + row] = l_tot > 0.f ? m_i + log2f(l_tot) : -INFINITY;
+        }
+        const int rows_valid = p.nq - first_row;
+        if (p.out_f32) {
+            constexpr int kPass = kTilesHere < D / 32 ? kTilesHere : D / 32;   // tiles per pass
+            float* ob = static_cast<float*>(p.o) + ((size_t)hz * p.nq + first_row) * D + col0;
+#pragma unroll
+            for (int h = 0; h < kTilesHere / kPass; ++h) {
+#pragma unroll
+                for (int i = 0; i < kPass; ++i) {
+                    const f32x4& acc = vals[h * kPass + i];
+                    const f32x4 val = {acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv};
+                    *reinterpret_cast<f32x4*>(stage + ql * kStageStride + (16 * i + 4 * g) * 4) = val;
+                }
+                __builtin_amdgcn_wave_barrier();
+                flush_rows<kPass * 64>(stage, kStageStride, reinterpret_cast<unsigned char*>(ob + h * kPass * 16),
+                                       (size_t)D * 4, lane, rows_valid);
+                __builtin_amdgcn_wave_barrier();
+            }
+        } else {
+            T* ob = static_cast<T*>(p.o) + ((size_t)hz * p.nq + first_row) * D + col0;
+#pragma unroll
+            for (int i = 0; i < kTilesHere; ++i) {
+                // accumulator rows 4g .. 4g+3 of a tile are 4 consecutive head dims
+                const f32x4& acc = vals[i];
+                const u32x2 packed = {MM::pack(acc[0] * inv, acc[1] * inv), MM::pack(acc[2] * inv, acc[3] * inv)};
+                *reinterpret_cast<u32x2*>(stage + ql * kStageStride + (16 * i + 4 * g) * 2) = packed;
+            }
+            __builtin_amdgcn_wave_barrier();
+            flush_rows<kTilesHere * 32>(stage, kStageStride, reinterpret_cast<unsigned char*>(ob), (size_t)D * 2, lane,
+                                        rows_valid);
+        }
+    };
+    if constexpr (kSplit == 1) {
+        __syncthreads();   // every wave is done with the last tile
+        finish(o, 0, smem + (size_t)qgroup * 16 * kStageStride, true);
+    } else {
+        // Two waves share each group of query rows: they swap halves of the head dimension
+        // through LDS (same lanes, same layout), and each merges, normalises and stores its half.
+        constexpr int kH = kDTiles / 2;
+        constexpr int kXchFloats = (2 + 4 * kH) * 64;
         __syncthreads();   // the ring is free: every tile has been consumed
-        float* xch = reinterpret_cast<float*>(smem) + (size_t)qgroup * (2 + 4 * kDTiles) * 64;
-        if (split == 1) {
-            xch[lane] = m_i;
-            xch[64 + lane] = l_i;
+        float* give = reinterpret_cast<float*>(smem) + (size_t)(qgroup * 2 + split) * kXchFloats;
+        const float* take = reinterpret_cast<float*>(smem) + (size_t)(qgroup * 2 + (1 - split)) * kXchFloats;
+        give[lane] = m_i;
+        give[64 + lane] = l_i;
+        f32x4 keep[kH];
+        if (split == 0) {
 #pragma unroll
-            for (int dt = 0; dt < kDTiles; ++dt)
+            for (int i = 0; i < kH; ++i) {
+                keep[i] = o[i];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) xch[(2 + 4 * dt + r) * 64 + lane] = o[dt][r];
+                for (int r = 0; r < 4; ++r) give[(2 + 4 * i + r) * 64 + lane] = o[kH + i][r];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kH; ++i) {
+                keep[i] = o[kH + i];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) give[(2 + 4 * i + r) * 64 + lane] = o[i][r];
+            }
         }
         __syncthreads();
-        if (split != 0) return;
-        const float m_b = xch[lane], l_b = xch[64 + lane];
+        const float m_b = take[lane], l_b = take[64 + lane];
         const float m_new = fmaxf(m_i, m_b);
         const float m_safe = m_new == -INFINITY ? 0.f : m_new;
         const float a_own = __builtin_amdgcn_exp2f(m_i - m_safe);
@@ -556,73 +642,11 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
         l_i = l_i * a_own + l_b * a_oth;
         m_i = m_new;
 #pragma unroll
-        for (int dt = 0; dt < kDTiles; ++dt)
+        for (int i = 0; i < kH; ++i)
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-                o[dt][r] = o[dt][r] * a_own + xch[(2 + 4 * dt + r) * 64 + lane] * a_oth;
-    }
-
-    // ---- epilogue: normalise, write O once (and the base-2 log-sum-exp) --------
-    const float l_tot = sum_quarters(l_i);
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    {
-        // the row number is derived again from an opaque copy: kept from the start-up it would
-        // occupy a register pair through the whole kernel
-        int rib = row_in_block;
-        asm volatile("" : "+v"(rib));
-        const int row = j * M + rib;
-        if (row < p.nq && p.lse && g == 0)
-            p.lse[(size_t)hz * p.nq + row] = l_tot > 0.f ? m_i + log2f(l_tot) : -INFINITY;
-    }
-    // In the accumulator layout 16 neighbouring lanes hold 16 different rows of O, which the
-    // memory pipeline would write as 64 separate 8-byte pieces per instruction.  The wave
-    // turns its 16 x D block around in LDS instead (the ring is free by now) and stores whole
-    // rows, 16 bytes per lane.  A float32 output goes in two column halves of the same size.
-    constexpr int kStageStride = D * 2 + 16;     // bytes per staged row (padded against bank conflicts)
-    constexpr int kLanesPerRow = D * 2 / 16;
-    constexpr int kRowsPerStore = 64 / kLanesPerRow;
-    constexpr int kStoreIters = 16 / kRowsPerStore;
-    unsigned char* stage;
-    if (kSplit > 1) {
-        stage = smem + (size_t)qgroup * (2 + 4 * kDTiles) * 64 * 4;   // own exchange area, already read
-    } else {
-        __syncthreads();   // every wave is done with the last tile
-        stage = smem + (size_t)qgroup * 16 * kStageStride;
-    }
-    const int st_row = lane / kLanesPerRow, st_piece = lane % kLanesPerRow;
-    const int first_row = j * M + qgroup * 16;
-    auto flush = [&](unsigned char* dst, size_t pitch) {   // dst: row first_row, first staged column
-#pragma unroll
-        for (int i = 0; i < kStoreIters; ++i) {
-            const int r = i * kRowsPerStore + st_row;
-            const u32x4 val = *reinterpret_cast<const u32x4*>(stage + r * kStageStride + st_piece * 16);
-            if (first_row + r < p.nq) *reinterpret_cast<u32x4*>(dst + r * pitch + st_piece * 16) = val;
-        }
-    };
-    if (p.out_f32) {
-        float* ob = static_cast<float*>(p.o) + ((size_t)hz * p.nq + first_row) * D;
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-#pragma unroll
-            for (int i = 0; i < kDTiles / 2; ++i) {
-                const int dt = h * (kDTiles / 2) + i;
-                const f32x4 val = {o[dt][0] * inv, o[dt][1] * inv, o[dt][2] * inv, o[dt][3] * inv};
-                *reinterpret_cast<f32x4*>(stage + ql * kStageStride + (16 * i + 4 * g) * 4) = val;
-            }
-            __builtin_amdgcn_wave_barrier();
-            flush(reinterpret_cast<unsigned char*>(ob + h * (D / 2)), (size_t)D * 4);
-            __builtin_amdgcn_wave_barrier();
-        }
-    } else {
-        T* ob = static_cast<T*>(p.o) + ((size_t)hz * p.nq + first_row) * D;
-#pragma unroll
-        for (int dt = 0; dt < kDTiles; ++dt) {
-            // accumulator rows 4g .. 4g+3 of tile dt are 4 consecutive head dims
-            const u32x2 packed = {MM::pack(o[dt][0] * inv, o[dt][1] * inv), MM::pack(o[dt][2] * inv, o[dt][3] * inv)};
-            *reinterpret_cast<u32x2*>(stage + ql * kStageStride + (16 * dt + 4 * g) * 2) = packed;
-        }
-        __builtin_amdgcn_wave_barrier();
-        flush(reinterpret_cast<unsigned char*>(ob), (size_t)D * 2);
+            for (int r = 0; r < 4; ++r) keep[i][r] = keep[i][r] * a_own + take[(2 + 4 * i + r) * 64 + lane] * a_oth;
+        unsigned char* stage = smem + (size_t)kQGroups * 2 * kXchFloats * 4 + (size_t)wave * 16 * kStageStride;
+        finish(keep, split * (D / 2), stage, split == 0);
     }
 }
 
@@ -639,7 +663,8 @@ int launch_ks(const AttnParams& p, hipStream_t stream) {
     if (stages < kQSlots + (M / 32 < 2 ? M / 32 : 2))
         return launch_attention_mfma(p, BF16 ? FSTA_BF16 : FSTA_F16, D, BF16 && !SPLIT, stream);
     // the epilogue reuses the front of the segment: exchange area of a key split, row staging
-    constexpr size_t kEpilogueBytes = KS > 1 ? (size_t)(M / 16) * (2 + D / 4) * 256 : (size_t)M * (D * 2 + 16);
+    constexpr size_t kEpilogueBytes = KS > 1 ? (size_t)(M / 16) * 2 * ((2 + D / 8) * 256 + 16 * (D * 2 + 16))
+                                             : (size_t)M * (D * 2 + 16);
     if (lds < kEpilogueBytes) lds = kEpilogueBytes;
     if (lds > 160 * 1024)
         return fail(FSTA_EUNSUPPORTED, "max_ancestors=%d needs %zu bytes of LDS (limit 163840)", p.max_anc, lds);
