@@ -232,7 +232,7 @@ def cpu_baseline(wl, budget_s=10.0):
     import torch
     from oracle import dense_attention, tree_precompute
     cores = os.cpu_count() or 1
-    cores = min(cores, 16) if "GRAFT_REPO_ROOT" in os.environ else cores
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))   # the share of the host this job owns
     torch.set_num_threads(cores)
     q, k, v, _ = wl.sets[0]
     heads = min(wl.h, 32)
@@ -296,7 +296,8 @@ def main():
     args = parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on one GPU (got --gpus {args.gpus}); the op shards over "
-              "batch*heads without communication, see DESIGN.md", file=sys.stderr)
+              "batch*heads without communication (every GPU would run this same launch on its share of "
+              "the heads)", file=sys.stderr)
         sys.exit(2)
     import torch
     if not torch.cuda.is_available():
