@@ -152,3 +152,43 @@ def renumber_parents_gpu(parent: torch.Tensor, perm: torch.Tensor, rank: torch.T
     """Parent array of the same forest after node ``perm[new]`` has been renamed ``new``."""
     old_parent = parent.index_select(0, perm)
     return torch.where(old_parent >= 0, rank.index_select(0, old_parent.clamp(min=0)), old_parent)
+
+
+def medusa_parents_gpu(probs: torch.Tensor, n: int) -> torch.Tensor:
+    """``probs [depths, topk]`` on the GPU -> parent array int64 ``[n]`` on the GPU, no host round trip.
+
+    Device version of ``trees.medusa_parents_from_probs`` (same selection, same tie-breaks, same
+    numbering): a path of ranks ``(r1..rd)`` scores the product of its ranks' probabilities, the
+    ``n-1`` best paths are kept (ties: shallower first, then smaller ranks) and numbered by
+    ``(depth, ranks)``; node 0 is the empty path.  Scores are formed in float64 in the host
+    version's multiplication order.  Plain torch tensor operations on the current stream; with
+    ``dfs_order_gpu``, ``lineage_from_parents_gpu(width=depths + 1)`` and
+    ``create_fst_attention_kernel_inputs(check=False)`` a tree goes from draft-head
+    probabilities to kernel inputs without touching the host.
+    """
+    if probs.dim() != 2 or not probs.is_cuda:
+        raise ValueError("probs must be a [depths, topk] tensor on the GPU")
+    depths, topk = probs.shape
+    total = sum(topk ** d for d in range(1, depths + 1))
+    if not 1 <= n <= total + 1:
+        raise ValueError(f"n={n} outside [1, {total + 1}] for depths={depths}, topk={topk}")
+    probs = probs.to(torch.float64)
+    dev = probs.device
+    # all paths in (depth, ranks) order: level d is the outer product of level d-1 with probs[d-1]
+    levels, score = [], torch.ones((1,), dtype=torch.float64, device=dev)
+    for d in range(depths):
+        score = (score[:, None] * probs[d][None, :]).reshape(-1)
+        levels.append(score)
+    scores = torch.cat(levels)                                   # key k -> path k + 1 in that order
+    best = torch.sort(scores, descending=True, stable=True).indices[: n - 1]   # stable: ties keep key order
+    kept = torch.sort(best).values + 1                           # keys of nodes 1 .. n-1 (key 0 = root)
+    # key -> (depth, value): value = ranks read as a base-topk number; the parent drops the last digit
+    starts = [1]
+    for d in range(1, depths + 1):
+        starts.append(starts[-1] + topk ** d)
+    bounds = torch.tensor(starts, dtype=torch.int64, device=dev)
+    level = torch.bucketize(kept, bounds, right=True) - 1        # 0-based depth index (depth - 1)
+    value = kept - bounds[level]
+    parent_key = torch.where(level > 0, bounds[(level - 1).clamp(min=0)] + value // topk, torch.zeros_like(kept))
+    parent_id = torch.where(parent_key > 0, torch.searchsorted(kept, parent_key) + 1, torch.zeros_like(kept))
+    return torch.cat([torch.full((1,), -1, dtype=torch.int64, device=dev), parent_id])

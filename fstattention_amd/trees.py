@@ -252,8 +252,19 @@ def medusa_parents(n: int = 256, depths: int = 4, topk: int = 10,
     ``(depth, ranks)``), numbered by ``(depth, ranks)`` ascending so that
     ``parent < child``.
     """
+    return medusa_parents_from_probs(medusa_probs(depths, topk, alpha, seed), n)
+
+
+def medusa_probs(depths: int = 4, topk: int = 10, alpha: float = 0.3, seed: int = 1002) -> np.ndarray:
+    """Seeded candidate probabilities ``[depths, topk]`` (float64), each row sorted descending."""
     rng = np.random.default_rng(seed)
-    probs = [np.sort(rng.dirichlet(alpha * np.ones(topk)))[::-1] for _ in range(depths)]
+    return np.stack([np.sort(rng.dirichlet(alpha * np.ones(topk)))[::-1] for _ in range(depths)])
+
+
+def medusa_parents_from_probs(probs, n: int) -> np.ndarray:
+    """Parent array of the tree of the ``n-1`` most probable paths for given ``probs [depths, topk]``."""
+    probs = np.asarray(probs, dtype=np.float64)
+    depths, topk = probs.shape
     cands = []
     for d in range(1, depths + 1):
         for ranks in itertools.product(range(topk), repeat=d):

@@ -5,7 +5,7 @@ import torch
 
 from conftest import golden_cases
 from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, lineage_from_parents_gpu,
-                              pack_tree_mask, renumber_parents_gpu, trees)
+                              medusa_parents_gpu, pack_tree_mask, renumber_parents_gpu, trees)
 from oracle import tree_precompute as tp
 
 pytestmark = pytest.mark.gpu
@@ -175,3 +175,30 @@ def test_dfs_order_on_gpu_flags_bad_parents_and_sizes():
         dfs_order_gpu(torch.full((16385,), -1, dtype=torch.int64).cuda())
     empty, _ = dfs_order_gpu(torch.empty((0,), dtype=torch.int64).cuda())
     assert empty.numel() == 0
+
+
+def test_medusa_tree_built_on_the_gpu_matches_the_host_builder():
+    for seed, depths, topk, n in [(1002, 4, 10, 256), (7, 4, 10, 64), (8, 3, 5, 100), (9, 2, 4, 21), (10, 4, 10, 1)]:
+        probs = trees.medusa_probs(depths, topk, 0.3, seed)
+        want = trees.medusa_parents_from_probs(probs, n)
+        got = medusa_parents_gpu(torch.from_numpy(probs).cuda(), n)
+        np.testing.assert_array_equal(got.cpu().numpy(), want)
+    with pytest.raises(ValueError):
+        medusa_parents_gpu(torch.ones((2, 3)).cuda(), 14)     # only 3 + 9 paths + root exist
+
+
+def test_device_only_pipeline_from_probabilities_to_kernel_inputs():
+    """probabilities -> tree -> depth-first order -> lineage -> kernel inputs, all on the device,
+    against the host chain on the same probabilities."""
+    probs = trees.medusa_probs(4, 10, 0.3, 1002)
+    parent = medusa_parents_gpu(torch.from_numpy(probs).cuda(), 256)
+    perm, rank = dfs_order_gpu(parent, "light_first", check=False)
+    new_parent = renumber_parents_gpu(parent, perm, rank)
+    lineage, level = lineage_from_parents_gpu(new_parent, width=5, check=False)
+    *got, status = create_fst_attention_kernel_inputs(lineage, level, 64, 64, check=False)
+    assert int(status.item()) == 0
+    host_parent = trees.medusa_parents_from_probs(probs, 256)
+    host_new, _ = trees.renumber_parents(host_parent, trees.dfs_order(host_parent, "light_first"))
+    lin, lvl = trees.lineage_from_parents(host_new, min_width=5)
+    want = tp.block_inputs(lin.numpy().copy(), lvl.numpy(), 64, 64)
+    _check(got, want)

@@ -177,3 +177,10 @@ def test_renumber_rejects_bad_orders():
         trees.renumber_parents(parent, np.array([1, 0, 2, 3]))   # child before parent
     with pytest.raises(ValueError):
         trees.dfs_order(parent, children="random")
+
+
+def test_medusa_builder_split_keeps_the_benchmark_tree():
+    probs = trees.medusa_probs(4, 10, 0.3, 1002)
+    assert probs.shape == (4, 10) and (np.diff(probs, axis=1) <= 0).all()
+    np.testing.assert_allclose(probs.sum(axis=1), 1.0)
+    np.testing.assert_array_equal(trees.medusa_parents_from_probs(probs, 256), trees.config(2).parent)
