@@ -103,6 +103,9 @@ class Workload:
         self.pairs = int(depth.sum() + self.n)
         self.flops = 4 * self.d * self.z * self.h * self.pairs
 
+        # HBM bytes a launch has to move at least once when nothing is cached from before:
+        # every K and V row, Q, O and the log-sum-exp (rows shared by blocks come from L2)
+        self.min_traffic_bytes = self.z * self.h * self.n * (4 * self.d * self.esz + 4)
         per_set = 4 * self.z * self.h * self.n * self.d * self.esz
         self.per_set_bytes = per_set
         self.n_sets = max(2, min(256, -(-sets_bytes // per_set)))
@@ -286,10 +289,16 @@ def copy_calibration(mib):
     src = torch.empty(n, dtype=torch.uint8, device="cuda").fill_(1)
     dst = torch.empty_like(src)
     torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
     for _ in range(10):
         dst.copy_(src)
+    ev1.record()
     torch.cuda.synchronize()
-    print(json.dumps({"copy_bytes": n, "copies": 10}))
+    seconds = ev0.elapsed_time(ev1) * 1e-3 / 10
+    # read + write traffic of a plain copy: what this box's HBM delivers to a streaming kernel
+    print(json.dumps({"copy_bytes": n, "copies": 10, "us_per_copy": round(seconds * 1e6, 1),
+                      "read_plus_write_gbps": round(2 * n / seconds / 1e9, 1)}))
 
 
 def main():
@@ -383,6 +392,8 @@ def main():
                 "kv_bytes_per_call": w.kv_bytes, "kv_gbps_cold": round(w.kv_bytes / ks / 1e9, 1),
                 "hbm_frac": round(w.kv_bytes / ks / 1e9 / HBM_PEAK_GBPS, 4),
                 "effective_tflops": round(w.flops / ks / 1e12, 3),
+                "q_k_v_o_bytes_once": w.min_traffic_bytes,
+                "q_k_v_o_gbps_cold": round(w.min_traffic_bytes / ks / 1e9, 1),
                 "gpu_precompute_us": round(time_precompute(w) * 1e6, 2),
                 "cross_check_ok": ok_i, "max_abs_diff_vs_scalar_kernel": err_i,
                 "batch": w.z, "heads": w.h, "max_ancestors": w.max_anc,
@@ -413,6 +424,8 @@ def main():
                 "us_per_call_cold": round(ti["cold_us"], 2), "kv_rows_per_head": w.kv_rows,
                 "kv_bytes_per_call": w.kv_bytes, "kv_gbps_cold": round(w.kv_bytes / ks / 1e9, 1),
                 "hbm_frac": round(w.kv_bytes / ks / 1e9 / HBM_PEAK_GBPS, 4),
+                "q_k_v_o_bytes_once": w.min_traffic_bytes,
+                "q_k_v_o_gbps_cold": round(w.min_traffic_bytes / ks / 1e9, 1),
                 "cross_check_ok": ok_i, "max_abs_diff_vs_scalar_kernel": err_i, "max_ancestors": w.max_anc,
             }
             del w
