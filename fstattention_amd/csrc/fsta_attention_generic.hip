@@ -165,11 +165,9 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
 template <typename T, int D, int M>
 int launch_one(const AttnParams& p, hipStream_t stream) {
     constexpr size_t lds = generic_lds_bytes<D, M>();
-    static bool configured = false;  // benign race: the call is idempotent
-    if (!configured) {
-        FSTA_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_generic_kernel<T, D, M>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        configured = true;
+    if (lds > 64 * 1024) {
+        const int rc = allow_full_lds<&attn_generic_kernel<T, D, M>>();
+        if (rc != FSTA_OK) return rc;
     }
     dim3 grid(p.nb, p.heads_total);
     hipLaunchKernelGGL((attn_generic_kernel<T, D, M>), grid, dim3(kThreads), lds, stream, p);

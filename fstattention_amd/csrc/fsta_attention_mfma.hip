@@ -487,9 +487,10 @@ int launch_one(const AttnParams& p, hipStream_t stream) {
     while (lds > 160 * 1024 && stages > 2) lds = mfma_lds_bytes<D, M>(p.max_anc, --stages);
     if (lds > 160 * 1024)
         return fail(FSTA_EUNSUPPORTED, "max_ancestors=%d needs %zu bytes of LDS (limit 163840)", p.max_anc, lds);
-    if (lds > 64 * 1024)
-        FSTA_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_mfma_kernel<BF16, D, M, SPLIT>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    if (lds > 64 * 1024) {
+        const int rc = allow_full_lds<&attn_mfma_kernel<BF16, D, M, SPLIT>>();
+        if (rc != FSTA_OK) return rc;
+    }
     const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
     const unsigned grid = (unsigned)(kXcds * slices_per_xcd * p.nb);
     hipLaunchKernelGGL((attn_mfma_kernel<BF16, D, M, SPLIT>), dim3(grid), dim3(M * 2 * key_split_for(M)), lds,

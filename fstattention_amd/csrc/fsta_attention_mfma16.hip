@@ -674,9 +674,10 @@ int launch_ks(const AttnParams& p, hipStream_t stream) {
     constexpr size_t kQBytes = (size_t)kWaves * 16 * D * 2;
     const int early = grid <= kCus && lds + kQBytes <= 160 * 1024 ? 1 : 0;
     if (early) lds += kQBytes;
-    if (lds > 64 * 1024)
-        FSTA_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_mfma16_kernel<BF16, D, M, SPLIT, KS>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    if (lds > 64 * 1024) {
+        const int rc = allow_full_lds<&attn_mfma16_kernel<BF16, D, M, SPLIT, KS>>();
+        if (rc != FSTA_OK) return rc;
+    }
     hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT, KS>), dim3(grid), dim3(M * 4 * KS), lds, stream, p,
                        stages, early);
     FSTA_HIP_OK(hipGetLastError());

@@ -40,6 +40,21 @@ int fail(int code, const char* fmt, ...);
             return ::fsta::fail(FSTA_EHIP, "%s: %s", #expr, hipGetErrorString(err__)); \
     } while (0)
 
+// Raises the dynamic-LDS limit of one kernel to the 160 KB of a gfx950 CU, once per device and
+// process (the attribute call costs microseconds on the host; setting it twice in a race is harmless).
+template <auto Kernel>
+int allow_full_lds() {
+    static bool done[64] = {};
+    int dev = 0;
+    FSTA_HIP_OK(hipGetDevice(&dev));
+    const bool tracked = dev >= 0 && dev < 64;
+    if (tracked && done[dev]) return FSTA_OK;
+    FSTA_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    160 * 1024));
+    if (tracked) done[dev] = true;
+    return FSTA_OK;
+}
+
 // launchers, one per translation unit
 int launch_attention_generic(const AttnParams& p, int dtype, int head_dim, hipStream_t stream);
 int launch_attention_mfma(const AttnParams& p, int dtype, int head_dim, bool fast_pv,

@@ -245,8 +245,10 @@ extern "C" int fsta_precompute(int64_t* lineage, const int64_t* level_lookup, in
         return fail(FSTA_EUNSUPPORTED,
                     "fsta_precompute: n_nodes=%lld block_m=%d max_ancestors=%d need %zu bytes of LDS (limit 163840)",
                     (long long)n_nodes, block_m, max_ancestors, lds);
-    FSTA_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(&block_precompute_kernel),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    if (lds > 64 * 1024) {
+        const int rc = allow_full_lds<&block_precompute_kernel>();
+        if (rc != FSTA_OK) return rc;
+    }
     const int64_t nb = (n_nodes + block_m - 1) / block_m;
     hipLaunchKernelGGL(block_precompute_kernel, dim3((unsigned)nb), dim3(kThreads), lds,
                        static_cast<hipStream_t>(stream), lineage, level_lookup, n_nodes, width,
