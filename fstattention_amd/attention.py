@@ -28,7 +28,31 @@ class PackedTreeMask(NamedTuple):
 
 
 def _stream_ptr(device) -> int:
-    return torch.cuda.current_stream(device).cuda_stream
+    """Raw handle of torch's current stream on `device` (the C accessor; the Python stream object
+    costs several microseconds per call)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    try:
+        return torch._C._cuda_getCurrentRawStream(index)
+    except AttributeError:      # accessor missing in this torch build
+        return torch.cuda.current_stream(device).cuda_stream
+
+
+class _on_device:
+    """``with`` block that makes `device` current only when it is not already."""
+
+    def __init__(self, device):
+        self.index = device.index
+        self.prev = None
+
+    def __enter__(self):
+        if self.index is not None and self.index != torch.cuda.current_device():
+            self.prev = torch.cuda.current_device()
+            torch.cuda.set_device(self.index)
+
+    def __exit__(self, *exc):
+        if self.prev is not None:
+            torch.cuda.set_device(self.prev)
+        return False
 
 
 def pack_tree_mask(ancestor_idx: torch.Tensor, ancestor_mask: torch.Tensor) -> PackedTreeMask:
@@ -49,7 +73,7 @@ def pack_tree_mask(ancestor_idx: torch.Tensor, ancestor_mask: torch.Tensor) -> P
     words = (a + 31) // 32
     bits = torch.empty((nb, words, m), dtype=torch.int32, device=dev)
     count = torch.empty((nb,), dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _lib.check(lib.fsta_pack_mask(ancestor_idx.data_ptr(), ancestor_mask.data_ptr(), nb, m, a,
                                       bits.data_ptr(), count.data_ptr(), _stream_ptr(dev)))
     return PackedTreeMask(bits, count, m, a)
@@ -144,12 +168,13 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
     leaf_idx = leaf_idx.contiguous()
     packed = _packed_for(ancestor_idx, ancestor_mask)
     o = torch.empty(q.shape, dtype=out_dtype, device=q.device)
-    lse = torch.empty((Z * H, Nq), device=q.device, dtype=torch.float32)
+    # the reference allocates L and drops it (fstattention.py:158-160,181); here it only exists when asked for
+    lse = torch.empty((Z * H, Nq), device=q.device, dtype=torch.float32) if return_lse else None
     flags = (_lib.FLAG_FAST_PV if fast_pv else 0) | (_lib.FLAG_GENERIC if generic else 0) | \
         (_lib.FLAG_WIDE_WAVES if wide_waves else 0)
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         _lib.check(lib.fsta_attention_fwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr() if return_lse else None,
             ancestor_idx.data_ptr(), packed.mask_bits.data_ptr(), packed.anc_count.data_ptr(),
             leaf_idx.data_ptr(), Z, H, Nq, Nk, D, _DTYPES[q.dtype], _DTYPES[out_dtype],
             BLOCK_M, MAX_ANCESTORS, nb, float(sm_scale), flags, _stream_ptr(q.device)))
@@ -193,7 +218,7 @@ def merge_attention_states(o_a: torch.Tensor, lse_a: torch.Tensor, o_b: torch.Te
     o_a, o_b, lse_a, lse_b = o_a.contiguous(), o_b.contiguous(), lse_a.contiguous(), lse_b.contiguous()
     o = torch.empty_like(o_a)
     lse = torch.empty_like(lse_a)
-    with torch.cuda.device(o_a.device):
+    with _on_device(o_a.device):
         _lib.check(lib.fsta_merge_states(o_a.data_ptr(), lse_a.data_ptr(), o_b.data_ptr(), lse_b.data_ptr(),
                                          o.data_ptr(), lse.data_ptr(), rows, d, _DTYPES[o_a.dtype],
                                          _stream_ptr(o_a.device)))

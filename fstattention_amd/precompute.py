@@ -11,7 +11,7 @@ from typing import Optional
 import torch
 
 from . import _lib
-from .attention import PackedTreeMask, _stream_ptr
+from .attention import PackedTreeMask, _on_device, _stream_ptr
 
 
 def _raise_for_status(status: int, max_ancestors: int):
@@ -68,7 +68,7 @@ def create_fst_attention_kernel_inputs(lineage, level_lookup, block_m=64, max_an
     bits = torch.empty((nb, words, block_m), dtype=torch.int32, device=dev)
     count = torch.empty((nb,), dtype=torch.int32, device=dev)
     status = torch.zeros((1,), dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _lib.check(lib.fsta_precompute(
             lin.data_ptr(), lvl.data_ptr(), n, width, block_m, max_ancestors, int(mutate_lineage),
             a_idx.data_ptr(), a_mask.data_ptr() if want_bool_mask else None, l_idx.data_ptr(),
@@ -102,7 +102,7 @@ def lineage_from_parents_gpu(parent: torch.Tensor, width: Optional[int] = None, 
     n = parent.shape[0]
     level = torch.empty((n,), dtype=torch.int64, device=dev)
     status = torch.zeros((1,), dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         if width is None:
             _lib.check(lib.fsta_lineage_from_parents(parent.data_ptr(), n, 1, None, level.data_ptr(),
                                                      status.data_ptr(), _stream_ptr(dev)))
@@ -139,7 +139,7 @@ def dfs_order_gpu(parent: torch.Tensor, children: str = "index", check: bool = T
     rank = torch.empty((n,), dtype=torch.int64, device=dev)
     work = torch.empty((2 * n,), dtype=torch.int32, device=dev)
     status = torch.zeros((1,), dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _lib.check(lib.fsta_dfs_order(parent.data_ptr(), n, 1 if children == "light_first" else 0,
                                       perm.data_ptr(), rank.data_ptr(), work.data_ptr(),
                                       status.data_ptr(), _stream_ptr(dev)))
