@@ -67,7 +67,7 @@ __device__ __forceinline__ void flush_rows(const unsigned char* stage, int strid
 // KS = waves that share one group of 16 query rows, each taking every KS-th tile with its own
 // running softmax (merged through LDS at the end).
 template <bool BF16, int D, int M, bool SPLIT, int KS>
-__global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p, int stages, int early_leaf) {
+__global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p, int stages, int early_leaf, int sub_shift) {
     using MM = Mma<BF16>;
     using T = typename MM::elem;
     using T2 = typename MM::elem2;
@@ -104,8 +104,15 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     // query blocks of a slice share one L2 for the K/V rows they have in common.
     const int xcd = blockIdx.x % kXcds;
     const int within = blockIdx.x / kXcds;
-    const int hz = (within / p.nb) * kXcds + xcd;
-    const int j = within % p.nb;
+    // A workgroup takes M consecutive rows: a whole block of the caller's, or (sub_shift = 1, small
+    // grids) one half of a block of 2M rows, so that twice as many CUs share the launch.  The
+    // half-block reads the block's ancestor list and its own rows of the mask and leaf list.
+    const int parts = p.nb << sub_shift;
+    const int hz = (within / parts) * kXcds + xcd;
+    const int part = within % parts;
+    const int j = part >> sub_shift;                                        // block of the caller's lists
+    const int block_rows = M << sub_shift;                                  // rows per such block
+    const int row_base = j * block_rows + (part & ((1 << sub_shift) - 1)) * M;   // first query row of this workgroup
     if (hz >= p.heads_total) return;
 
     const int tid = threadIdx.x;
@@ -116,7 +123,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     const int ql = lane & 15;        // query (column of S^T / O^T) of this lane
     const int g = lane >> 4;         // which quarter of the rows of an accumulator tile
     const int row_in_block = qgroup * 16 + ql;
-    const int qrow = j * M + row_in_block;
+    const int qrow = row_base + row_in_block;
 
     const T* qb = static_cast<const T*>(p.q) + (size_t)hz * p.nq * D;
     const T* kb = static_cast<const T*>(p.k) + (size_t)hz * p.nk * D;
@@ -130,12 +137,16 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     int n_anc = p.anc_count ? p.anc_count[j] : p.max_anc;
     // mask words: straight global->LDS copy, 16 bytes per lane, 1 KiB pieces dealt to the waves
     {
-        const int mask_bytes = p.mask_words * M * 4;   // multiple of 128
-        const char* src = reinterpret_cast<const char*>(p.mask_bits) + (size_t)j * mask_bytes;
-        for (int piece = wave; piece * 1024 < mask_bytes; piece += kWaves) {
-            if (piece * 1024 + lane * 16 < mask_bytes)
+        // source: [word][block_rows] words of block j, of which this workgroup takes M per word
+        const int chunks = p.mask_words * (M / 4);     // 16-byte pieces
+        const char* src = reinterpret_cast<const char*>(p.mask_bits) +
+                          ((size_t)j * p.mask_words * block_rows + (row_base - j * block_rows)) * 4;
+        for (int piece = wave; piece * 64 < chunks; piece += kWaves) {
+            const int c = piece * 64 + lane;
+            if (c < chunks)
                 __builtin_amdgcn_global_load_lds(
-                    (const void __attribute__((address_space(1)))*)(src + piece * 1024 + lane * 16),
+                    (const void __attribute__((address_space(1)))*)(src + ((size_t)(c / (M / 4)) * block_rows * 4 +
+                                                                           (c % (M / 4)) * 16)),
                     (void __attribute__((address_space(3)))*)(reinterpret_cast<char*>(mask_s) + piece * 1024),
                     16, 0, 0);
         }
@@ -147,7 +158,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
 #pragma unroll
         for (int i = 0; i < kKeyBatch; ++i) {
             const int c = c0 + i * kThreads;
-            const int64_t* src = c < M ? p.leaf_idx + (size_t)j * M + c
+            const int64_t* src = c < M ? p.leaf_idx + (size_t)row_base + c
                                        : p.ancestor_idx + (size_t)j * p.max_anc + min(c - M, p.max_anc - 1);
             raw[i] = global_read_b64(src);
         }
@@ -160,7 +171,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
             ids[i] = c - M < p.max_anc ? (int64_t)(((uint64_t)raw[i][1] << 32) | raw[i][0]) : -1;
         }
     };
-    u32x2 leaf_raw = global_read_b64(p.leaf_idx + (size_t)j * M + row_in_block);
+    u32x2 leaf_raw = global_read_b64(p.leaf_idx + (size_t)row_base + row_in_block);
     u32x2 first_raw[kKeyBatch];
     load_ids(tid, first_raw);
     // Q rows of this wave: whole rows straight into LDS, K-tile swizzle, parked in the last ring
@@ -177,7 +188,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
 #pragma unroll
     for (int i = 0; i < kQDma; ++i) {
         const int r = i * kRowsPerDma + dma_row;
-        const int grow = min(j * M + qgroup * 16 + r, p.nq - 1);
+        const int grow = min(row_base + qgroup * 16 + r, p.nq - 1);
         __builtin_amdgcn_global_load_lds(
             (const void __attribute__((address_space(1)))*)(qb + (size_t)grow * D + k_chunk<D>(r, dma_slot) * 8),
             (void __attribute__((address_space(3)))*)(qstage + i * 512), 16, 0, 0);
@@ -221,7 +232,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
         int rows[kRowGroups];
 #pragma unroll
         for (int i = 0; i < kRowGroups; ++i)
-            rows[i] = min(p.prefix + j * M + t * kTileN + ((wave * kDmaPerWave) / 2 + i) * kRowsPerDma + dma_row, p.nk - 1);
+            rows[i] = min(p.prefix + row_base + t * kTileN + ((wave * kDmaPerWave) / 2 + i) * kRowsPerDma + dma_row, p.nk - 1);
         issue_rows(t, t, rows);
     }
 
@@ -559,7 +570,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     // its block around in LDS instead (the ring is free by now) and stores whole rows, 16 bytes
     // per lane; columns go in passes of at most 2*D bytes per row.
     constexpr int kStageStride = D * 2 + 16;     // bytes per staged row (padded against bank conflicts)
-    const int first_row = j * M + qgroup * 16;
+    const int first_row = row_base + qgroup * 16;
     auto finish = [&](auto& vals, int col0, unsigned char* stage, bool write_lse) {
         constexpr int kTilesHere = (int)(sizeof(vals) / sizeof(vals[0]));
         const float l_tot = sum_quarters(l_i);
@@ -569,7 +580,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
             // would occupy a register pair through the whole kernel
             int rib = row_in_block;
             asm volatile("" : "+v"(rib));
-            const int row = j * M + rib;
+            const int row = row_base + rib;
             if (row < p.nq && p.lse && g == 0)
                 p.lse[(size_t)hz * p.nq + row] = l_tot > 0.f ? m_i + log2f(l_tot) : -INFINITY;
         }
@@ -651,7 +662,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
 }
 
 template <bool BF16, int D, int M, bool SPLIT, int KS>
-int launch_ks(const AttnParams& p, hipStream_t stream) {
+int launch_ks(const AttnParams& p, int sub_shift, hipStream_t stream) {
     // ring depth: everything in flight at once for short tile lists, else the limit
     const int tiles = M / 32 + anc_tile_capacity(p.max_anc) + (p.prefix + kTileN - 1) / kTileN;
     int stages = tiles < 2 ? 2 : (tiles > kMaxStages ? kMaxStages : tiles);
@@ -669,7 +680,7 @@ int launch_ks(const AttnParams& p, hipStream_t stream) {
     if (lds > 160 * 1024)
         return fail(FSTA_EUNSUPPORTED, "max_ancestors=%d needs %zu bytes of LDS (limit 163840)", p.max_anc, lds);
     const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
-    const unsigned grid = (unsigned)(kXcds * slices_per_xcd * p.nb);
+    const unsigned grid = (unsigned)(kXcds * slices_per_xcd * (p.nb << sub_shift));
     // a launch whose workgroups all run at once: leaf tiles requested early, Q in an area of its own
     constexpr size_t kQBytes = (size_t)kWaves * 16 * D * 2;
     const int early = grid <= kCus && lds + kQBytes <= 160 * 1024 ? 1 : 0;
@@ -679,28 +690,31 @@ int launch_ks(const AttnParams& p, hipStream_t stream) {
         if (rc != FSTA_OK) return rc;
     }
     hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT, KS>), dim3(grid), dim3(M * 4 * KS), lds, stream, p,
-                       stages, early);
+                       stages, early, sub_shift);
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
 }
 
 template <bool BF16, int D, int M, bool SPLIT>
-int launch_one(const AttnParams& p, hipStream_t stream) {
+int launch_one(const AttnParams& p, int sub_shift, hipStream_t stream) {
     // Key splitting pays when a wave would otherwise walk several ancestor / prefix tiles on
     // its own and the block is small (few waves); blocks of 128 rows fill the workgroup anyway.
     const int work_tiles = anc_tile_capacity(p.max_anc) + (p.prefix + kTileN - 1) / kTileN;
     if constexpr (M < 128) {
-        if (work_tiles >= 2) return launch_ks<BF16, D, M, SPLIT, 2>(p, stream);
+        if (work_tiles >= 2) return launch_ks<BF16, D, M, SPLIT, 2>(p, sub_shift, stream);
     }
-    return launch_ks<BF16, D, M, SPLIT, 1>(p, stream);
+    return launch_ks<BF16, D, M, SPLIT, 1>(p, sub_shift, stream);
 }
 
 template <bool BF16, int D, bool SPLIT>
 int launch_m(const AttnParams& p, hipStream_t stream) {
+    // Launches that would leave half of the CUs without a workgroup are cut into half-blocks.
+    const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
+    const bool halve = kXcds * slices_per_xcd * p.nb * 2 <= kCus;
     switch (p.block_m) {
-        case 32: return launch_one<BF16, D, 32, SPLIT>(p, stream);
-        case 64: return launch_one<BF16, D, 64, SPLIT>(p, stream);
-        case 128: return launch_one<BF16, D, 128, SPLIT>(p, stream);
+        case 32: return launch_one<BF16, D, 32, SPLIT>(p, 0, stream);
+        case 64: return halve ? launch_one<BF16, D, 32, SPLIT>(p, 1, stream) : launch_one<BF16, D, 64, SPLIT>(p, 0, stream);
+        case 128: return halve ? launch_one<BF16, D, 64, SPLIT>(p, 1, stream) : launch_one<BF16, D, 128, SPLIT>(p, 0, stream);
     }
     return fail(FSTA_EUNSUPPORTED, "matrix-core kernel: block_m=%d", p.block_m);
 }
