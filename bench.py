@@ -57,6 +57,8 @@ def parse_args():
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="instead of the benchmark, run 10 device-to-device copies of MIB MiB "
                          "(reference point for the FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--dtype", choices=["bf16", "f16", "f32"], default=None,
+                    help="storage type of q/k/v (default: the configuration's own, bf16 for the headline)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-graph", action="store_true", help="time plain stream launches only")
     return ap.parse_args()
@@ -318,7 +320,8 @@ def main():
         return
     use_graph = not args.no_graph
 
-    wl = Workload(args.config, sets_bytes=2 * INFINITY_CACHE_BYTES)
+    dtype = {None: None, "bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[args.dtype]
+    wl = Workload(args.config, sets_bytes=2 * INFINITY_CACHE_BYTES, dtype=dtype)
     ok, max_err, tol = wl.cross_check()
     if not ok:
         print(f"bench.py: the two kernels disagree (max difference {max_err:.3e} > {tol})", file=sys.stderr)

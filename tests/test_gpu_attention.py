@@ -320,6 +320,29 @@ def test_prefix_and_tree_parts_merge_into_the_full_result(dtype):
         merge_attention_states(o_t, l_t[:, :5], o_p, l_p)
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes_against_oracle(seed):
+    """Seeded draw over tree shape, size (ragged last blocks included), block size, head dim,
+    storage type, prefix length and slice count; every fourth case has enough slices for several
+    rounds of workgroups per CU (the start-up differs between small and large launches)."""
+    rng = np.random.default_rng(1000 + seed)
+    block_m = int(rng.choice([32, 64, 128]))
+    d = int(rng.choice([32, 64, 128]))
+    dtype = [torch.bfloat16, torch.float16][seed % 2]
+    n = int(rng.integers(1, 5 * block_m))
+    kind = seed % 3
+    if kind == 0:
+        parent = trees.random_recursive_parents(n, seed)
+    elif kind == 1:
+        parent = trees.random_recursive_parents(n, seed, window=int(rng.integers(1, 9)))   # deep
+    else:
+        parent = np.maximum((np.arange(n) - 1) // int(rng.integers(2, 12)), -1).astype(np.int64)   # bushy
+        parent[0] = -1
+    prefix = int(rng.choice([0, 0, int(rng.integers(1, 150))]))
+    z, h = (2, 72) if seed % 4 == 3 else (int(rng.integers(1, 3)), int(rng.integers(1, 4)))
+    run_tree(parent, block_m, z, h, d, dtype, seed, prefix=prefix, wide_waves=(seed % 8 == 5))
+
+
 def test_rows_without_any_key_give_zero():
     a_idx = torch.full((1, 8), -1, dtype=torch.int64)
     a_mask = torch.zeros((1, 16, 8), dtype=torch.bool)
