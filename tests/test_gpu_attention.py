@@ -343,6 +343,79 @@ def test_random_shapes_against_oracle(seed):
     run_tree(parent, block_m, z, h, d, dtype, seed, prefix=prefix, wide_waves=(seed % 8 == 5))
 
 
+def test_hip_graph_replays_match_eager_calls():
+    """The op captured into a HIP graph (precompute + attention, as a decoding step would), replayed
+    several times with eager launches and synchronisations in between; every replay must give the
+    eager result for the inputs its buffers hold at that moment."""
+    cfg = trees.config(2)
+    m, d = cfg.block_m, cfg.head_dim
+    lineage, level = trees.lineage_from_parents(cfg.parent)
+    lineage, level = lineage.cuda(), level.cuda()
+    max_anc = trees.required_max_ancestors(cfg.parent, m)
+    scale = 1.0 / math.sqrt(d)
+    q, k, v = (t.cuda() for t in rand_qkv(1, 4, cfg.n_nodes, cfg.n_nodes, d, cfg.dtype, 31))
+
+    def step():
+        *inputs, _ = create_fst_attention_kernel_inputs(lineage, level, m, max_anc, mutate_lineage=False,
+                                                        check=False, want_bool_mask=False)
+        return fst_attention(q, k, v, *inputs, scale, BLOCK_M=m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32)
+
+    eager = step().clone()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        step()
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            out = step()
+    for replay in range(4):
+        if replay:                                   # new inputs in the same buffers, eager work in between
+            g = torch.Generator().manual_seed(100 + replay)
+            q.copy_(torch.randn(q.shape, generator=g).to(q.dtype))
+            eager = step().clone()
+            torch.cuda.synchronize()
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {replay} differs from the eager call"
+    want, _ = dense_oracle(q.cpu(), k.cpu(), v.cpu(), cfg.parent, scale)
+    assert_close(out, want, cfg.dtype, "last replay")
+
+
+def test_two_host_threads_on_their_own_streams():
+    """Entry points keep no state between calls: two threads, each with its own stream, inputs and
+    tree, launching at the same time get their own results."""
+    import threading
+    cases, results, errors = [], {}, []
+    for tid, (index, seed) in enumerate([(2, 1), (3, 2)]):
+        cfg = trees.config(index)
+        a_idx, a_mask, l_idx, max_anc = oracle_inputs(cfg.parent, cfg.block_m)
+        q, k, v = rand_qkv(1, 2, cfg.n_nodes, cfg.n_nodes, cfg.head_dim, cfg.dtype, seed)
+        want, _ = dense_oracle(q, k, v, cfg.parent, 0.1)
+        cases.append((tid, cfg, [t.cuda() for t in (q, k, v, a_idx, a_mask, l_idx)], max_anc, want))
+    torch.cuda.synchronize()
+
+    def work(tid, cfg, dev, max_anc):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(25):
+                    o = fst_attention(*dev, 0.1, BLOCK_M=cfg.block_m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32)
+            stream.synchronize()
+            results[tid] = o
+        except Exception as exc:   # surfaced by the assertion below
+            errors.append(exc)
+
+    threads = [threading.Thread(target=work, args=c[:4]) for c in cases]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for tid, cfg, _, _, want in cases:
+        assert_close(results[tid], want, cfg.dtype, f"thread {tid}")
+
+
 def test_rows_without_any_key_give_zero():
     a_idx = torch.full((1, 8), -1, dtype=torch.int64)
     a_mask = torch.zeros((1, 16, 8), dtype=torch.bool)
