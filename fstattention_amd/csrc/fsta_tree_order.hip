@@ -15,7 +15,7 @@ namespace fsta {
 namespace {
 
 constexpr int kOrderThreads = 256;
-constexpr int kSiblingTile = 1024;   // candidate siblings staged in LDS per step
+constexpr int kSiblingTile = 256;    // candidate siblings staged in LDS per workgroup
 
 __device__ __forceinline__ int32_t load_coherent(const int32_t* p) {
     // values produced by atomics of other workgroups: read past this CU's L1
@@ -30,21 +30,37 @@ __global__ __launch_bounds__(kOrderThreads) void order_init_kernel(int64_t n, in
     }
 }
 
-// Every hop must go to a smaller id (or to -1), so the walks below end whatever the input holds.
+// The walks to the root are chains of dependent reads; every workgroup first copies the parent
+// array (as int32; n <= 16384) into LDS so that a hop costs an LDS access, not a trip to L2.
+// Every hop must go to a smaller id (or to -1), so the walks end whatever the input holds.
+__device__ __forceinline__ void stage_parents(const int64_t* __restrict__ parent, int64_t n, int32_t* par_s) {
+    for (int64_t i = threadIdx.x; i < n; i += kOrderThreads) {
+        const int64_t p = parent[i];
+        par_s[i] = (p >= -1 && p < i) ? (int32_t)p : -2;   // -2: malformed entry
+    }
+    __syncthreads();
+}
+
+// Every node adds 1 to each of its ancestors.  All nodes meet at the roots, so the counts are
+// first gathered per workgroup in LDS and only the non-zero sums go to the global array.
 __global__ __launch_bounds__(kOrderThreads) void order_sizes_kernel(const int64_t* __restrict__ parent, int64_t n,
                                                                     int32_t* size, uint32_t* status) {
+    extern __shared__ int32_t par_s[];       // [n] parents, then [n] counts of this workgroup
+    int32_t* count_s = par_s + n;
+    for (int64_t x = threadIdx.x; x < n; x += kOrderThreads) count_s[x] = 0;
+    stage_parents(parent, n, par_s);
     const int64_t i = (int64_t)blockIdx.x * kOrderThreads + threadIdx.x;
-    if (i >= n) return;
-    int64_t cur = i, p = parent[i];
-    while (p != -1) {
-        if (p < -1 || p >= cur) {
-            atomicOr(status, FSTA_PRE_BAD_NODE_ID);
-            return;
+    if (i < n) {
+        int32_t p = par_s[i];
+        while (p >= 0) {
+            atomicAdd(&count_s[p], 1);
+            p = par_s[p];
         }
-        atomicAdd(&size[p], 1);
-        cur = p;
-        p = parent[cur];
+        if (p < -1) atomicOr(status, FSTA_PRE_BAD_NODE_ID);
     }
+    __syncthreads();
+    for (int64_t x = threadIdx.x; x < n; x += kOrderThreads)
+        if (count_s[x]) atomicAdd(&size[x], count_s[x]);
 }
 
 // grid (ceil(n / kOrderThreads), ceil(n / kSiblingTile)): thread i against the candidates of tile y
@@ -53,14 +69,13 @@ __global__ __launch_bounds__(kOrderThreads) void order_siblings_kernel(const int
                                                                        int32_t* off) {
     __shared__ int32_t par_s[kSiblingTile];
     __shared__ int32_t size_s[kSiblingTile];
-    const int64_t i = (int64_t)blockIdx.x * kOrderThreads + threadIdx.x;
-    const int64_t s0 = (int64_t)blockIdx.y * kSiblingTile;
+    const int i = blockIdx.x * kOrderThreads + threadIdx.x;       // n <= 16384: 32-bit arithmetic throughout
+    const int s0 = blockIdx.y * kSiblingTile;
     // a sibling has an id above the common parent; with plain index order it also lies below i
-    const int64_t block_first = (int64_t)blockIdx.x * kOrderThreads;
-    const int64_t block_last = min(block_first + kOrderThreads, n) - 1;
+    const int block_last = min((int)(blockIdx.x + 1) * kOrderThreads, (int)n) - 1;
     if (!light_first && s0 > block_last) return;
     for (int t = threadIdx.x; t < kSiblingTile; t += kOrderThreads) {
-        const int64_t s = s0 + t;
+        const int s = s0 + t;
         par_s[t] = s < n ? (int32_t)parent[s] : -2;     // -2 never matches
         size_s[t] = s < n ? load_coherent(size + s) : 0;
     }
@@ -68,13 +83,19 @@ __global__ __launch_bounds__(kOrderThreads) void order_siblings_kernel(const int
     if (i >= n) return;
     const int32_t my_parent = (int32_t)parent[i];
     const int32_t my_size = load_coherent(size + i);
-    const int count = (int)min((int64_t)kSiblingTile, n - s0);
+    const int count = min(kSiblingTile, (int)n - s0);
     int32_t acc = 0;
-    for (int t = 0; t < count; ++t) {
-        const int64_t s = s0 + t;
-        const bool sibling = par_s[t] == my_parent && s != i;
-        const bool before = light_first ? (size_s[t] < my_size || (size_s[t] == my_size && s < i)) : s < i;
-        acc += (sibling && before) ? size_s[t] : 0;
+    if (light_first) {
+        // order key (size, id) packed into one comparison: sizes and ids are below 2^15
+        const int32_t my_key = (my_size << 15) | i;
+#pragma unroll 4
+        for (int t = 0; t < count; ++t) {
+            const int32_t key = (size_s[t] << 15) | (s0 + t);
+            acc += (par_s[t] == my_parent && key < my_key) ? size_s[t] : 0;
+        }
+    } else {
+#pragma unroll 4
+        for (int t = 0; t < count; ++t) acc += (par_s[t] == my_parent && s0 + t < i) ? size_s[t] : 0;
     }
     if (acc) atomicAdd(&off[i], acc);
 }
@@ -83,20 +104,21 @@ __global__ __launch_bounds__(kOrderThreads) void order_finish_kernel(const int64
                                                                      const int32_t* off, int64_t* __restrict__ perm,
                                                                      int64_t* __restrict__ rank,
                                                                      const uint32_t* status) {
+    extern __shared__ int32_t par_s[];       // [n] parents, then [n] sibling offsets
+    int32_t* off_s = par_s + n;
     const int64_t i = (int64_t)blockIdx.x * kOrderThreads + threadIdx.x;
-    if (i >= n) return;
     if (*status) {      // malformed parent array: identity, the caller reads the status word
-        perm[i] = i;
-        rank[i] = i;
+        if (i < n) {
+            perm[i] = i;
+            rank[i] = i;
+        }
         return;
     }
-    int64_t pre = -1, cur = i;
-    while (cur >= 0) {
-        pre += load_coherent(off + cur) + 1;
-        const int64_t p = parent[cur];
-        if (p >= cur) break;
-        cur = p;
-    }
+    for (int64_t x = threadIdx.x; x < n; x += kOrderThreads) off_s[x] = load_coherent(off + x);
+    stage_parents(parent, n, par_s);
+    if (i >= n) return;
+    int64_t pre = -1;
+    for (int32_t cur = (int32_t)i; cur >= 0; cur = par_s[cur]) pre += off_s[cur] + 1;
     perm[pre] = i;
     rank[i] = pre;
 }
@@ -120,12 +142,19 @@ extern "C" int fsta_dfs_order(const int64_t* parent, int64_t n_nodes, int32_t li
     int32_t* off = workspace + n_nodes;
     const unsigned blocks = (unsigned)((n_nodes + kOrderThreads - 1) / kOrderThreads);
     const unsigned tiles = (unsigned)((n_nodes + kSiblingTile - 1) / kSiblingTile);
+    const size_t lds_parents = (size_t)n_nodes * sizeof(int32_t);
+    if (2 * lds_parents > 64 * 1024) {
+        int rc = allow_full_lds<&order_sizes_kernel>();
+        if (rc == FSTA_OK) rc = allow_full_lds<&order_finish_kernel>();
+        if (rc != FSTA_OK) return rc;
+    }
     hipLaunchKernelGGL(order_init_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, n_nodes, size, off);
-    hipLaunchKernelGGL(order_sizes_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, parent, n_nodes, size, status);
+    hipLaunchKernelGGL(order_sizes_kernel, dim3(blocks), dim3(kOrderThreads), 2 * lds_parents, s, parent, n_nodes,
+                       size, status);
     hipLaunchKernelGGL(order_siblings_kernel, dim3(blocks, tiles), dim3(kOrderThreads), 0, s, parent, n_nodes,
                        light_first ? 1 : 0, size, off);
-    hipLaunchKernelGGL(order_finish_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, parent, n_nodes, off, perm,
-                       rank, status);
+    hipLaunchKernelGGL(order_finish_kernel, dim3(blocks), dim3(kOrderThreads), 2 * lds_parents, s, parent, n_nodes,
+                       off, perm, rank, status);
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
 }
