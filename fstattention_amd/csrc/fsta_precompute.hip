@@ -184,36 +184,50 @@ __global__ __launch_bounds__(kThreads) void pack_mask_kernel(
     if (tid == 0) anc_count[j] = last_valid + 1;
 }
 
+// `lds_nodes` > 0: the workgroup first copies parent[0 .. lds_nodes) into LDS as int32 (the walks to
+// the root are chains of dependent reads: an LDS access per hop instead of a trip to L2).
 __global__ __launch_bounds__(kThreads) void lineage_from_parents_kernel(
     const int64_t* __restrict__ parent, int64_t n_nodes, int64_t width,
     int64_t* __restrict__ lineage, int64_t* __restrict__ level_lookup,
-    uint32_t* __restrict__ status) {
-    const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    uint32_t* __restrict__ status, int lds_nodes) {
+    extern __shared__ int32_t par_s[];
+    for (int x = threadIdx.x; x < lds_nodes; x += kThreads) {
+        const int64_t v = parent[x];
+        par_s[x] = (v >= -1 && v < x) ? (int32_t)v : -2;   // -2: malformed entry
+    }
+    const int64_t first = (int64_t)blockIdx.x * kThreads;
+    const int64_t last = min(first + kThreads, n_nodes);
+    if (lineage) {   // the rows of this workgroup's nodes are one contiguous piece: fill it with -1, coalesced
+        int64_t* piece = lineage + first * width;
+        for (int64_t e = threadIdx.x; e < (last - first) * width; e += kThreads) piece[e] = -1;
+    }
+    __syncthreads();
+    const int64_t i = first + threadIdx.x;
     if (i >= n_nodes) return;
+    auto up = [&](int64_t node) -> int64_t {   // parent of `node`, or -2 for an entry outside [-1, node)
+        if (lds_nodes) return par_s[node];
+        const int64_t v = parent[node];
+        return (v >= -1 && v < node) ? v : -2;
+    };
     uint32_t err = 0u;
-    // pass 1: depth of node i; every hop must go to a smaller id, so the walk ends
+    // pass 1: depth of node i; every hop goes to a smaller id, so the walk ends
     int64_t depth = 0;
-    int64_t p = parent[i], cur = i;
-    while (p != -1) {
-        if (p < -1 || p >= cur) { err |= FSTA_PRE_BAD_NODE_ID; break; }
+    for (int64_t a = up(i); a != -1; a = up(a)) {
+        if (a < -1) { err |= FSTA_PRE_BAD_NODE_ID; break; }
         ++depth;
-        cur = p;
-        p = parent[cur];
     }
     level_lookup[i] = depth;
-    if (!lineage) {  // levels only
-        if (err) atomicOr(status, err);
-        return;
-    }
-    int64_t* row = lineage + i * width;
-    for (int64_t l = 0; l < width; ++l) row[l] = -1;
-    if (!err && depth >= width) err |= FSTA_PRE_BAD_LEVEL;
-    if (!err) {
-        // pass 2: the ancestor reached after s hops lives at level depth - s
-        int64_t a = parent[i];
-        for (int64_t l = depth - 1; l >= 0; --l) {
-            row[l] = a;
-            a = parent[a];
+    if (lineage && !err) {
+        if (depth >= width) {
+            err |= FSTA_PRE_BAD_LEVEL;
+        } else {
+            // pass 2: the ancestor reached after s hops lives at level depth - s
+            int64_t* row = lineage + i * width;
+            int64_t a = up(i);
+            for (int64_t l = depth - 1; l >= 0; --l) {
+                row[l] = a;
+                a = up(a);
+            }
         }
     }
     if (err) atomicOr(status, err);
@@ -284,9 +298,10 @@ extern "C" int fsta_lineage_from_parents(const int64_t* parent, int64_t n_nodes,
     if (!parent || !level_lookup || !status)
         return fail(FSTA_EINVAL, "fsta_lineage_from_parents: null pointer");
     const unsigned grid = (unsigned)((n_nodes + kThreads - 1) / kThreads);
-    hipLaunchKernelGGL(lineage_from_parents_kernel, dim3(grid), dim3(kThreads), 0,
+    const int lds_nodes = n_nodes <= 16384 ? (int)n_nodes : 0;   // 64 KB of int32
+    hipLaunchKernelGGL(lineage_from_parents_kernel, dim3(grid), dim3(kThreads), (size_t)lds_nodes * 4,
                        static_cast<hipStream_t>(stream), parent, n_nodes, width, lineage,
-                       level_lookup, status);
+                       level_lookup, status, lds_nodes);
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
 }
