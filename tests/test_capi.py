@@ -69,6 +69,12 @@ def test_argument_validation_happens_before_any_gpu_work():
     assert lib.fsta_pack_mask(None, None, 0, 16, 8, None, None, None) == _lib.OK
     assert lib.fsta_pack_mask(None, None, 2, 16, 0, None, None, None) == _lib.EINVAL
     assert lib.fsta_lineage_from_parents(None, 5, 0, None, None, None, None) == _lib.EINVAL
+    assert lib.fsta_dfs_order(None, -1, 0, None, None, None, None, None) == _lib.EINVAL
+    assert lib.fsta_dfs_order(None, 1 << 20, 0, None, None, None, None, None) == _lib.EUNSUPPORTED
+    assert lib.fsta_dfs_order(None, 8, 0, None, None, None, None, None) == _lib.EINVAL      # null pointers
+    assert lib.fsta_merge_states(None, None, None, None, None, None, 4, 12, _lib.BF16, None) == _lib.EINVAL   # head dim
+    assert lib.fsta_merge_states(None, None, None, None, None, None, 4, 64, 7, None) == _lib.EINVAL          # null pointers come first
+    assert lib.fsta_merge_states(None, None, None, None, None, None, 0, 64, _lib.BF16, None) == _lib.OK       # nothing to do
     with pytest.raises(_lib.FstaError):
         _lib.check(_lib.EINVAL)
 
@@ -82,6 +88,14 @@ def test_python_entry_points_refuse_to_run_without_a_gpu_path():
     leaf = torch.arange(16).view(1, 16)
     with pytest.raises(ValueError, match="GPU"):
         fst_attention(q, q, q, idx, mask, leaf, 1.0, BLOCK_M=16, MAX_ANCESTORS=8)
+    from fstattention_amd import dfs_order_gpu, medusa_parents_gpu, merge_attention_states
+    lse = torch.zeros(16)
+    with pytest.raises(ValueError, match="GPU"):
+        merge_attention_states(q, lse, q, lse)
+    with pytest.raises(ValueError, match="GPU"):
+        dfs_order_gpu(torch.tensor([-1, 0], dtype=torch.int64))
+    with pytest.raises(ValueError, match="GPU"):
+        medusa_parents_gpu(torch.ones(2, 3), 4)
     if not torch.cuda.is_available():
         lineage, level = trees.lineage_from_parents([-1, 0, 1])
         with pytest.raises(RuntimeError, match="GPU"):
