@@ -67,9 +67,10 @@ def parse_args():
 class Workload:
     """Device-resident inputs of one configuration, in `sets` rotating copies."""
 
-    def __init__(self, index, sets_bytes, dtype=None, heads=None, batch=None, order=None):
+    def __init__(self, index, sets_bytes, dtype=None, heads=None, batch=None, order=None, prefix=0,
+                 key_splits=None):
         import torch
-        from fstattention_amd import _lib, create_fst_attention_kernel_inputs, trees
+        from fstattention_amd import _lib, create_fst_attention_kernel_inputs, shift_for_prefix, trees
         from fstattention_amd.attention import _DTYPES, _packed_for
 
         self.torch = torch
@@ -96,30 +97,42 @@ class Workload:
         self.max_anc = trees.required_max_ancestors(cfg.parent, self.m, 16)
         self.a_idx, self.a_mask, self.l_idx = create_fst_attention_kernel_inputs(
             self.lineage, self.level, self.m, self.max_anc, mutate_lineage=False)
+        # K/V laid out as [shared prefix | tree] (reference fstattention.py:209-212)
+        self.prefix = prefix
+        self.nk = self.n + prefix
+        if prefix:
+            self.a_idx, self.l_idx = shift_for_prefix(self.a_idx, self.l_idx, prefix)
         self.packed = _packed_for(self.a_idx, self.a_mask)
         self.nb = self.a_idx.shape[0]
         rows = int((self.a_idx >= 0).sum().item() + (self.l_idx >= 0).sum().item())
-        self.kv_rows = rows
-        self.kv_bytes = self.z * self.h * 2 * self.d * self.esz * rows
+        self.kv_rows = rows + self.nb * prefix       # every block walks the whole prefix
+        self.kv_bytes = self.z * self.h * 2 * self.d * self.esz * self.kv_rows
         depth = trees.levels_from_parents(cfg.parent)
-        self.pairs = int(depth.sum() + self.n)
+        self.pairs = int(depth.sum() + self.n) + self.n * prefix
         self.flops = 4 * self.d * self.z * self.h * self.pairs
 
         # HBM bytes a launch has to move at least once when nothing is cached from before:
         # every K and V row, Q, O and the log-sum-exp (rows shared by blocks come from L2)
-        self.min_traffic_bytes = self.z * self.h * self.n * (4 * self.d * self.esz + 4)
-        per_set = 4 * self.z * self.h * self.n * self.d * self.esz
+        self.min_traffic_bytes = self.z * self.h * ((2 * self.n + 2 * self.nk) * self.d * self.esz + 4 * self.n)
+        per_set = self.z * self.h * (2 * self.n + 2 * self.nk) * self.d * self.esz
         self.per_set_bytes = per_set
         self.n_sets = max(2, min(256, -(-sets_bytes // per_set)))
         shape = (self.z, self.h, self.n, self.d)
+        kv_shape = (self.z, self.h, self.nk, self.d)
+        # workspace for a prefix cut into runs of keys (none wanted: plain entry point)
+        self.flags = _lib.flag_key_splits(key_splits) if key_splits else 0
+        need = self.lib.fsta_attention_workspace_bytes(self.z, self.h, self.n, self.nk, self.d, self.code, self.m,
+                                                       self.max_anc, self.scale, self.flags) if prefix else 0
+        self.key_runs = need // (self.z * self.h * self.n * (self.d + 1) * 4) if need else 1
+        self.work = torch.empty((need,), dtype=torch.uint8, device=dev) if need else None
         g = torch.Generator().manual_seed(cfg.tensor_seed)
         self.sets = []
         base = None
         for s in range(self.n_sets):
             if s < 4 or base is None:
                 # CPU-seeded N(0,1), rounded to the storage type, then moved
-                q, k, v = (torch.randn(shape, generator=g, dtype=torch.float32).to(cfg.dtype).to(dev)
-                           for _ in range(3))
+                q, k, v = (torch.randn(sh, generator=g, dtype=torch.float32).to(cfg.dtype).to(dev)
+                           for sh in (shape, kv_shape, kv_shape))
                 base = (q, k, v)
             else:
                 # further sets: device-side copies rolled along the sequence axis (distinct
@@ -133,11 +146,20 @@ class Workload:
         """One step: a single call through the C ABI on torch's current stream."""
         torch = self.torch
         q, k, v, o = self.sets[s % self.n_sets]
+        if self.work is not None:
+            self._check(self.lib.fsta_attention_fwd_ws(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), self.lse.data_ptr(),
+                self.a_idx.data_ptr(), self.packed.mask_bits.data_ptr(), self.packed.anc_count.data_ptr(),
+                self.l_idx.data_ptr(), self.z, self.h, self.n, self.nk, self.d, self.code, self.code,
+                self.m, self.max_anc, self.nb, self.scale, flags | self.flags, self.work.data_ptr(),
+                self.work.numel(), torch.cuda.current_stream().cuda_stream))
+            return
         self._check(self.lib.fsta_attention_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), self.lse.data_ptr(),
             self.a_idx.data_ptr(), self.packed.mask_bits.data_ptr(), self.packed.anc_count.data_ptr(),
-            self.l_idx.data_ptr(), self.z, self.h, self.n, self.n, self.d, self.code, self.code,
-            self.m, self.max_anc, self.nb, self.scale, flags, torch.cuda.current_stream().cuda_stream))
+            self.l_idx.data_ptr(), self.z, self.h, self.n, self.nk, self.d, self.code, self.code,
+            self.m, self.max_anc, self.nb, self.scale, flags | self.flags,
+            torch.cuda.current_stream().cuda_stream))
 
     def run_default(self, heads):
         """float32 output of the default kernel on the first `heads` slices of set 0."""
@@ -434,6 +456,26 @@ def main():
             }
             del w
             torch.cuda.empty_cache()
+        # the headline tree behind a shared prefix (the KV cache of a decoding step, reference
+        # fstattention.py:113-136): the prefix as each block's own loop, and cut into runs of keys
+        for prefix in (4096, 16384):
+            entry = {}
+            for label, forced in (("one_launch", 1), ("key_runs", None)):
+                w = Workload(2, sets_bytes=2 * INFINITY_CACHE_BYTES, prefix=prefix, key_splits=forced)
+                ok_i, err_i, _ = w.cross_check()
+                ti = summarize(w, max(20, min(args.steps, 100)), min(args.warmup, 10), use_graph, False)
+                ks = ti["cold_event_us"] * 1e-6
+                entry[label] = {
+                    "us_per_call_cold": round(ti["cold_us"], 2), "key_runs": int(w.key_runs),
+                    "kv_bytes_per_call": w.kv_bytes, "kv_gbps_cold": round(w.kv_bytes / ks / 1e9, 1),
+                    "q_k_v_o_bytes_once": w.min_traffic_bytes,
+                    "q_k_v_o_gbps_cold": round(w.min_traffic_bytes / ks / 1e9, 1),
+                    "effective_tflops": round(w.flops / ks / 1e12, 1),
+                    "cross_check_ok": ok_i, "max_abs_diff_vs_scalar_kernel": err_i,
+                }
+                del w
+                torch.cuda.empty_cache()
+            extra[f"medusa256_behind_prefix_{prefix}"] = entry
         result["extra"] = extra
     print(json.dumps(result))
 

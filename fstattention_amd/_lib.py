@@ -3,13 +3,20 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_uint32, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_uint32, c_void_p
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libfsta.so")
 
 F32, F16, BF16 = 0, 1, 2
 OK, EINVAL, EUNSUPPORTED, EHIP = 0, -1, -2, -3
 FLAG_FAST_PV, FLAG_GENERIC, FLAG_WIDE_WAVES = 1, 2, 4
+
+
+def flag_key_splits(n: int) -> int:
+    """FSTA_FLAG_KEY_SPLITS(n): force n runs of prefix keys (1 = never split, 0 = library decides)."""
+    return (int(n) & 0xFF) << 8
+
+
 PRE_TOO_MANY_ANCESTORS, PRE_BAD_NODE_ID, PRE_BAD_LEVEL = 1, 2, 4
 ABI_VERSION = 1
 
@@ -26,6 +33,12 @@ SIGNATURES = {
                                    c_void_p, c_void_p, c_void_p, c_void_p,
                                    c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
                                    c_int32, c_int32, c_int32, c_float, c_uint32, c_void_p]),
+    "fsta_attention_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
+                                                  c_int32, c_float, c_uint32]),
+    "fsta_attention_fwd_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                      c_void_p, c_void_p, c_void_p, c_void_p,
+                                      c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
+                                      c_int32, c_int32, c_int32, c_float, c_uint32, c_void_p, c_size_t, c_void_p]),
     "fsta_lineage_from_parents": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
                                           c_void_p]),
     "fsta_dfs_order": (c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,

@@ -105,7 +105,7 @@ def _packed_for(ancestor_idx: torch.Tensor, ancestor_mask) -> PackedTreeMask:
 def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
                   BLOCK_M=128, MAX_ANCESTORS=64, *, out_dtype: Optional[torch.dtype] = None,
                   return_lse: bool = False, fast_pv: bool = False, generic: bool = False,
-                  wide_waves: bool = False):
+                  wide_waves: bool = False, key_splits: Optional[int] = None):
     """Fused sparse tree attention forward (reference ``fstattention.py:153-181``).
 
     ``q [Z,H,Nq,D]``, ``k,v [Z,H,Nk,D]`` (``Nk - Nq`` leading rows are a dense
@@ -119,7 +119,10 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
     the reference computes and drops (``fstattention.py:139-141,181``),
     ``fast_pv`` trades accuracy of the bf16 weights for matrix-core time,
     ``generic`` forces the scalar kernel and ``wide_waves`` the matrix-core variant
-    with 32 instead of 16 query rows per wave.  Inputs the reference silently
+    with 32 instead of 16 query rows per wave.  A long shared prefix in front of few
+    query blocks is cut into runs of keys that separate workgroups take (the partial
+    results live in a temporary workspace and are joined by a second kernel);
+    ``key_splits`` forces the number of runs (``1``: never split).  Inputs the reference silently
     mis-handles raise ``ValueError`` here (non-contiguous tensors, index
     tensors whose shapes do not match ``BLOCK_M`` / ``MAX_ANCESTORS``).
     """
@@ -171,13 +174,21 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
     # the reference allocates L and drops it (fstattention.py:158-160,181); here it only exists when asked for
     lse = torch.empty((Z * H, Nq), device=q.device, dtype=torch.float32) if return_lse else None
     flags = (_lib.FLAG_FAST_PV if fast_pv else 0) | (_lib.FLAG_GENERIC if generic else 0) | \
-        (_lib.FLAG_WIDE_WAVES if wide_waves else 0)
+        (_lib.FLAG_WIDE_WAVES if wide_waves else 0) | (_lib.flag_key_splits(key_splits) if key_splits else 0)
+    # a shared prefix may be worth cutting into key runs: the library says how much workspace that takes
+    work, work_bytes = None, 0
+    if Nk > Nq:
+        work_bytes = lib.fsta_attention_workspace_bytes(Z, H, Nq, Nk, D, _DTYPES[q.dtype], BLOCK_M,
+                                                        MAX_ANCESTORS, float(sm_scale), flags)
+        if work_bytes:
+            work = torch.empty((work_bytes,), dtype=torch.uint8, device=q.device)
     with _on_device(q.device):
-        _lib.check(lib.fsta_attention_fwd(
+        _lib.check(lib.fsta_attention_fwd_ws(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr() if return_lse else None,
             ancestor_idx.data_ptr(), packed.mask_bits.data_ptr(), packed.anc_count.data_ptr(),
             leaf_idx.data_ptr(), Z, H, Nq, Nk, D, _DTYPES[q.dtype], _DTYPES[out_dtype],
-            BLOCK_M, MAX_ANCESTORS, nb, float(sm_scale), flags, _stream_ptr(q.device)))
+            BLOCK_M, MAX_ANCESTORS, nb, float(sm_scale), flags,
+            work.data_ptr() if work is not None else None, work_bytes, _stream_ptr(q.device)))
     return (o, lse) if return_lse else o
 
 

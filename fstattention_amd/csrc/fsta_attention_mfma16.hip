@@ -66,7 +66,8 @@ __device__ __forceinline__ void flush_rows(const unsigned char* stage, int strid
 
 // KS = waves that share one group of 16 query rows, each taking every KS-th tile with its own
 // running softmax (merged through LDS at the end).
-template <bool BF16, int D, int M, bool SPLIT, int KS>
+// RUNS = the launch cuts the shared prefix into runs of keys (AttnParams::key_splits > 1).
+template <bool BF16, int D, int M, bool SPLIT, int KS, bool RUNS>
 __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p, int stages, int early_leaf, int sub_shift) {
     using MM = Mma<BF16>;
     using T = typename MM::elem;
@@ -103,7 +104,16 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     // Workgroup -> (slice, block), XCD-aware: every XCD gets whole (batch, head) slices, so all
     // query blocks of a slice share one L2 for the K/V rows they have in common.
     const int xcd = blockIdx.x % kXcds;
-    const int within = blockIdx.x / kXcds;
+    int within = blockIdx.x / kXcds;
+    // Key splits (long shared prefix, few blocks): workgroup `ksp` of a block takes the ksp-th run
+    // of prefix tiles, workgroup 0 also the tree part; each writes a normalised partial result
+    // and its log-sum-exp, which a merge kernel joins.
+    int ksp = 0;
+    if constexpr (RUNS) {
+        ksp = within % p.key_splits;
+        within /= p.key_splits;
+    }
+    const bool tree = !RUNS || ksp == 0;
     // A workgroup takes M consecutive rows: a whole block of the caller's, or (sub_shift = 1, small
     // grids) one half of a block of 2M rows, so that twice as many CUs share the launch.  The
     // half-block reads the block's ancestor list and its own rows of the mask and leaf list.
@@ -268,7 +278,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     lds_tie(leaf_raw);
     const int64_t leaf64 = (int64_t)(((uint64_t)leaf_raw[1] << 32) | leaf_raw[0]);
     store_keys(tid, first_ids);
-    const bool leaf_ok = leaf64 >= 0 && leaf64 < p.nk;
+    const bool leaf_ok = tree && leaf64 >= 0 && leaf64 < p.nk;
     {   // does any valid leaf slot name another row than the one requested above?
         const bool other = leaf_ok && (row_in_block >> 5) < n_spec && leaf64 != (int64_t)p.prefix + qrow;
         if (lane == 0) lds_write_b32(lds_addr(spec_s + wave), 0u);
@@ -300,9 +310,15 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
         }
     };
     if (!early_leaf) read_q(0);   // Q sits in ring slots the gathers are about to take
-    n_anc = min(max(n_anc, 0), p.max_anc);
+    n_anc = tree ? min(max(n_anc, 0), p.max_anc) : 0;
     const int listed_tiles = kLeafTiles + (n_anc + kTileN - 1) / kTileN;
-    const int total_tiles = listed_tiles + (p.prefix + kTileN - 1) / kTileN;
+    int prefix_first = 0, prefix_end = (p.prefix + kTileN - 1) / kTileN;   // this workgroup's prefix tiles
+    if constexpr (RUNS) {
+        prefix_first = min(ksp * p.split_tiles, prefix_end);
+        prefix_end = min(prefix_first + p.split_tiles, prefix_end);
+    }
+    const int total_tiles = listed_tiles + prefix_end - prefix_first;
+    const int prefix_shift = prefix_first - listed_tiles;   // list position t holds prefix tile t + prefix_shift
     ring_barrier();
 
     auto issue = [&](int t, int slot) {
@@ -312,7 +328,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
         for (int i = 0; i < kRowGroups; ++i) {
             const int r = ((wave * kDmaPerWave) / 2 + i) * kRowsPerDma + dma_row;
             if (t < listed_tiles) rows[i] = key_s[t * kTileN + r];
-            else rows[i] = min((t - listed_tiles) * kTileN + r, p.prefix - 1);
+            else rows[i] = min((t + prefix_shift) * kTileN + r, p.prefix - 1);
         }
         issue_rows(t, slot, rows);
     };
@@ -323,6 +339,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     // order), barrier (everyone's share has landed, everyone is done with the tiles before),
     // then refill the slots that barrier freed.
     int issued = n_spec, issue_slot = n_spec, consumed = 0, slot = 0;   // n_spec < stages
+    if (!tree) issued = consumed = kLeafTiles;   // no tree part: the list starts behind the leaf tiles
     auto refill = [&]() {
         while (issued < total_tiles && issued < consumed + stages) {
             issue(issued, issue_slot);
@@ -354,12 +371,20 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     {   // a leaf list that names other rows than the ones requested: start the ring over
         const u32x4 f0 = lds_read_b128(lds_addr(spec_s)), f1 = lds_read_b128(lds_addr(spec_s + 4));
         lds_wait();
-        u32x4 any = f0 | f1;
-        lds_tie(any);
-        if (__builtin_amdgcn_readfirstlane(any[0] | any[1] | any[2] | any[3]) != 0u) {
+        u32x4 lo = f0, hi = f1;
+        lds_tie(lo);
+        lds_tie(hi);
+        uint32_t any = 0u;   // only the flags of waves that exist have been written
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const uint32_t a = lo[w], b = hi[w];
+            if (w < kWaves) any |= a;
+            if (w + 4 < kWaves) any |= b;
+        }
+        if (__builtin_amdgcn_readfirstlane(any) != 0u) {
             wait_vmcnt<0>();
             __syncthreads();
-            issued = 0;
+            issued = consumed;
             issue_slot = 0;
         }
     }
@@ -374,7 +399,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     // Leaf tile i = the block's own rows 32i .. 32i+31 (reference fstattention.py:86-91,104-107):
     // query r sees exactly row r of it.  The two waves owning those rows take one dot product
     // per query from it on the vector ALU and seed their running softmax with it.
-    for (int base = 0; base < kLeafTiles; base += kLeafGroup) {
+    for (int base = tree ? 0 : kLeafTiles; base < kLeafTiles; base += kLeafGroup) {
         begin_step(kLeafGroup);
         const int my_tile = qgroup >> 1;
         if (split == 0 && my_tile >= base && my_tile < base + kLeafGroup && __ballot(leaf_ok) != 0ull) {
@@ -444,7 +469,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
         if (t < listed_tiles) {
             word = mask_s[(t - kLeafTiles) * M + row_in_block] & valid_s[t];
         } else if (t < total_tiles) {
-            const int left = p.prefix - (t - listed_tiles) * kTileN;
+            const int left = p.prefix - (t + prefix_shift) * kTileN;
             word = left >= 32 ? 0xffffffffu : ((1u << left) - 1u);
         }
         if (kSplit > 1 && t >= total_tiles) continue;   // this share has no tile in the last step
@@ -571,6 +596,10 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     // per lane; columns go in passes of at most 2*D bytes per row.
     constexpr int kStageStride = D * 2 + 16;     // bytes per staged row (padded against bank conflicts)
     const int first_row = row_base + qgroup * 16;
+    const int hz_out = RUNS ? hz + ksp * p.heads_total : hz;
+    float* const lse_out = RUNS ? p.part_lse : p.lse;
+    void* const o_out = RUNS ? static_cast<void*>(p.part_o) : p.o;
+    const bool out_f32 = RUNS || p.out_f32;
     auto finish = [&](auto& vals, int col0, unsigned char* stage, bool write_lse) {
         constexpr int kTilesHere = (int)(sizeof(vals) / sizeof(vals[0]));
         const float l_tot = sum_quarters(l_i);
@@ -581,13 +610,13 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
             int rib = row_in_block;
             asm volatile("" : "+v"(rib));
             const int row = row_base + rib;
-            if (row < p.nq && p.lse && g == 0)
-                p.lse[(size_t)hz * p.nq + row] = l_tot > 0.f ? m_i + log2f(l_tot) : -INFINITY;
+            if (row < p.nq && lse_out && g == 0)
+                lse_out[(size_t)hz_out * p.nq + row] = l_tot > 0.f ? m_i + log2f(l_tot) : -INFINITY;
         }
         const int rows_valid = p.nq - first_row;
-        if (p.out_f32) {
+        if (out_f32) {
             constexpr int kPass = kTilesHere < D / 32 ? kTilesHere : D / 32;   // tiles per pass
-            float* ob = static_cast<float*>(p.o) + ((size_t)hz * p.nq + first_row) * D + col0;
+            float* ob = static_cast<float*>(o_out) + ((size_t)hz_out * p.nq + first_row) * D + col0;
 #pragma unroll
             for (int h = 0; h < kTilesHere / kPass; ++h) {
 #pragma unroll
@@ -602,7 +631,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
                 __builtin_amdgcn_wave_barrier();
             }
         } else {
-            T* ob = static_cast<T*>(p.o) + ((size_t)hz * p.nq + first_row) * D + col0;
+            T* ob = static_cast<T*>(o_out) + ((size_t)hz_out * p.nq + first_row) * D + col0;
 #pragma unroll
             for (int i = 0; i < kTilesHere; ++i) {
                 // accumulator rows 4g .. 4g+3 of a tile are 4 consecutive head dims
@@ -671,8 +700,10 @@ int launch_ks(const AttnParams& p, int sub_shift, hipStream_t stream) {
     // the kernel's start-up parks Q in the last ring slots and requests up to two leaf tiles
     // into the first ones; ancestor lists too long to leave that much LDS go to the other kernel
     constexpr int kWaves = M / 16 * KS, kQSlots = (kWaves * 16 + 2 * kTileN - 1) / (2 * kTileN);
-    if (stages < kQSlots + (M / 32 < 2 ? M / 32 : 2))
+    if (stages < kQSlots + (M / 32 < 2 ? M / 32 : 2)) {
+        if (p.key_splits > 1) return FSTA_EUNSUPPORTED;   // the caller falls back to a launch without key splits
         return launch_attention_mfma(p, BF16 ? FSTA_BF16 : FSTA_F16, D, BF16 && !SPLIT, stream);
+    }
     // the epilogue reuses the front of the segment: exchange area of a key split, row staging
     constexpr size_t kEpilogueBytes = KS > 1 ? (size_t)(M / 16) * 2 * ((2 + D / 8) * 256 + 16 * (D * 2 + 16))
                                              : (size_t)M * (D * 2 + 16);
@@ -680,17 +711,26 @@ int launch_ks(const AttnParams& p, int sub_shift, hipStream_t stream) {
     if (lds > 160 * 1024)
         return fail(FSTA_EUNSUPPORTED, "max_ancestors=%d needs %zu bytes of LDS (limit 163840)", p.max_anc, lds);
     const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
-    const unsigned grid = (unsigned)(kXcds * slices_per_xcd * (p.nb << sub_shift));
+    const unsigned grid = (unsigned)(kXcds * slices_per_xcd * (p.nb << sub_shift) * p.key_splits);
     // a launch whose workgroups all run at once: leaf tiles requested early, Q in an area of its own
     constexpr size_t kQBytes = (size_t)kWaves * 16 * D * 2;
-    const int early = grid <= kCus && lds + kQBytes <= 160 * 1024 ? 1 : 0;
+    const int early = grid <= kCus && p.key_splits == 1 && lds + kQBytes <= 160 * 1024 ? 1 : 0;
     if (early) lds += kQBytes;
-    if (lds > 64 * 1024) {
-        const int rc = allow_full_lds<&attn_mfma16_kernel<BF16, D, M, SPLIT, KS>>();
-        if (rc != FSTA_OK) return rc;
+    if (p.key_splits > 1) {
+        if (lds > 64 * 1024) {
+            const int rc = allow_full_lds<&attn_mfma16_kernel<BF16, D, M, SPLIT, KS, true>>();
+            if (rc != FSTA_OK) return rc;
+        }
+        hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT, KS, true>), dim3(grid), dim3(M * 4 * KS), lds,
+                           stream, p, stages, early, sub_shift);
+    } else {
+        if (lds > 64 * 1024) {
+            const int rc = allow_full_lds<&attn_mfma16_kernel<BF16, D, M, SPLIT, KS, false>>();
+            if (rc != FSTA_OK) return rc;
+        }
+        hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT, KS, false>), dim3(grid), dim3(M * 4 * KS), lds,
+                           stream, p, stages, early, sub_shift);
     }
-    hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT, KS>), dim3(grid), dim3(M * 4 * KS), lds, stream, p,
-                       stages, early, sub_shift);
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
 }
@@ -710,7 +750,7 @@ template <bool BF16, int D, bool SPLIT>
 int launch_m(const AttnParams& p, hipStream_t stream) {
     // Launches that would leave half of the CUs without a workgroup are cut into half-blocks.
     const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
-    const bool halve = kXcds * slices_per_xcd * p.nb * 2 <= kCus;
+    const bool halve = kXcds * slices_per_xcd * p.nb * 2 * p.key_splits <= kCus;
     switch (p.block_m) {
         case 32: return launch_one<BF16, D, 32, SPLIT>(p, 0, stream);
         case 64: return halve ? launch_one<BF16, D, 32, SPLIT>(p, 1, stream) : launch_one<BF16, D, 64, SPLIT>(p, 0, stream);

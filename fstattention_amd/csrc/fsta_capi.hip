@@ -24,6 +24,55 @@ extern "C" int fsta_abi_version(void) { return FSTA_ABI_VERSION; }
 
 extern "C" const char* fsta_last_error(void) { return g_error; }
 
+namespace {
+
+constexpr int kKeyTile = 32;        // keys per tile of the attention kernels
+constexpr int kMinRunTiles = 8;     // shortest run of prefix tiles worth a workgroup of its own
+constexpr int kTargetGroups = 512;  // two workgroups per CU
+
+// How the shared prefix is cut for a launch of the narrow matrix-core kernel: number of runs
+// (1 = no split) and prefix tiles per run.  Depends on the shape and flags only, so that the
+// workspace query and the launch agree.
+int plan_key_splits(int64_t slices, int nq, int nk, int head_dim, int dtype, int block_m, float sm_scale,
+                    uint32_t flags, int* split_tiles) {
+    const int tiles = (nk - nq + kKeyTile - 1) / kKeyTile;
+    *split_tiles = tiles;
+    if (tiles < 2 || slices <= 0 || nq <= 0) return 1;
+    if ((flags & (FSTA_FLAG_GENERIC | FSTA_FLAG_WIDE_WAVES)) || !(sm_scale > 0.f) ||
+        !mfma_supported(dtype, head_dim, block_m))
+        return 1;
+    const int forced = (int)((flags >> 8) & 0xffu);
+    int64_t want = forced;
+    if (!forced) {
+        const int64_t groups = ((slices + 7) / 8) * 8 * ((nq + block_m - 1) / block_m);
+        want = (kTargetGroups + groups - 1) / groups;
+        if (want > tiles / kMinRunTiles) want = tiles / kMinRunTiles;
+    }
+    if (want > tiles) want = tiles;
+    if (want > 255) want = 255;
+    if (want <= 1) return 1;
+    const int per = (int)((tiles + want - 1) / want);
+    *split_tiles = per;
+    return (tiles + per - 1) / per;
+}
+
+size_t key_split_bytes(int splits, int64_t slices, int nq, int head_dim) {
+    return (size_t)splits * (size_t)slices * (size_t)nq * (size_t)(head_dim + 1) * sizeof(float);
+}
+
+}  // namespace
+
+extern "C" size_t fsta_attention_workspace_bytes(int32_t batch, int32_t heads, int32_t nq, int32_t nk,
+                                                 int32_t head_dim, int32_t dtype, int32_t block_m,
+                                                 int32_t max_ancestors, float sm_scale, uint32_t flags) {
+    (void)max_ancestors;
+    if (batch <= 0 || heads <= 0 || nq <= 0 || nk <= nq || block_m <= 0) return 0;
+    int split_tiles = 0;
+    const int64_t slices = (int64_t)batch * heads;
+    const int splits = plan_key_splits(slices, nq, nk, head_dim, dtype, block_m, sm_scale, flags, &split_tiles);
+    return splits > 1 ? key_split_bytes(splits, slices, nq, head_dim) : 0;
+}
+
 extern "C" int fsta_attention_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                                   const int64_t* ancestor_idx, const uint32_t* mask_bits,
                                   const int32_t* anc_count, const int64_t* leaf_idx,
@@ -31,6 +80,19 @@ extern "C" int fsta_attention_fwd(const void* q, const void* k, const void* v, v
                                   int32_t head_dim, int32_t dtype, int32_t out_dtype,
                                   int32_t block_m, int32_t max_ancestors, int32_t num_blocks,
                                   float sm_scale, uint32_t flags, void* stream) {
+    return fsta_attention_fwd_ws(q, k, v, o, lse, ancestor_idx, mask_bits, anc_count, leaf_idx, batch, heads, nq,
+                                 nk, head_dim, dtype, out_dtype, block_m, max_ancestors, num_blocks, sm_scale,
+                                 flags, nullptr, 0, stream);
+}
+
+extern "C" int fsta_attention_fwd_ws(const void* q, const void* k, const void* v, void* o, float* lse,
+                                     const int64_t* ancestor_idx, const uint32_t* mask_bits,
+                                     const int32_t* anc_count, const int64_t* leaf_idx,
+                                     int32_t batch, int32_t heads, int32_t nq, int32_t nk,
+                                     int32_t head_dim, int32_t dtype, int32_t out_dtype,
+                                     int32_t block_m, int32_t max_ancestors, int32_t num_blocks,
+                                     float sm_scale, uint32_t flags, void* workspace, size_t workspace_bytes,
+                                     void* stream) {
     if (batch < 0 || heads < 0 || nq < 0 || nk < nq)
         return fail(FSTA_EINVAL, "fsta_attention_fwd: batch=%d heads=%d nq=%d nk=%d (need nk >= nq >= 0)",
                     batch, heads, nq, nk);
@@ -65,8 +127,27 @@ extern "C" int fsta_attention_fwd(const void* q, const void* k, const void* v, v
     p.heads_total = (int32_t)slices;
     p.out_f32 = (out_dtype == FSTA_F32) ? 1 : 0;
     p.scale_log2e = sm_scale * kLog2e;
+    p.key_splits = 1; p.split_tiles = 0; p.part_o = nullptr; p.part_lse = nullptr;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (workspace) {
+        int split_tiles = 0;
+        const int splits = plan_key_splits(slices, nq, nk, head_dim, dtype, block_m, sm_scale, flags, &split_tiles);
+        if (splits > 1 && workspace_bytes >= key_split_bytes(splits, slices, nq, head_dim)) {
+            if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+                return fail(FSTA_EINVAL, "fsta_attention_fwd_ws: workspace must be 16-byte aligned");
+            AttnParams ps = p;
+            ps.key_splits = splits;
+            ps.split_tiles = split_tiles;
+            ps.part_o = static_cast<float*>(workspace);
+            ps.part_lse = ps.part_o + (size_t)splits * slices * nq * head_dim;
+            const int rc = launch_attention_mfma16(ps, dtype, head_dim, (flags & FSTA_FLAG_FAST_PV) != 0, s);
+            if (rc == FSTA_OK)
+                return launch_merge_splits(ps.part_o, ps.part_lse, splits, slices * nq, head_dim, o, out_dtype, lse, s);
+            // (this shape cannot take the narrow kernel: one launch without key splits below)
+            if (rc != FSTA_EUNSUPPORTED) return rc;
+        }
+    }
     // the matrix-core kernel takes row maxima before scaling, which needs a positive scale
     if (!(flags & FSTA_FLAG_GENERIC) && sm_scale > 0.f && mfma_supported(dtype, head_dim, block_m)) {
         const bool fast_pv = (flags & FSTA_FLAG_FAST_PV) != 0;

@@ -28,6 +28,12 @@ struct AttnParams {
     int32_t heads_total;          // batch * heads
     int32_t out_f32;              // o is float32 instead of the input type
     float scale_log2e;            // sm_scale * log2(e)
+    // Key splits of the shared prefix (narrow matrix-core kernel only; 1 = off): workgroup s of a
+    // block takes prefix tiles [s * split_tiles, (s + 1) * split_tiles) and writes a normalised
+    // float32 partial result part_o[s][batch*heads][nq][D] with log-sum-exp part_lse[s][batch*heads][nq].
+    int32_t key_splits, split_tiles;
+    float* part_o;
+    float* part_lse;
 };
 
 // Records a message for fsta_last_error() and returns `code`.
@@ -62,6 +68,9 @@ int launch_attention_mfma(const AttnParams& p, int dtype, int head_dim, bool fas
 int launch_attention_mfma16(const AttnParams& p, int dtype, int head_dim, bool fast_pv,
                             hipStream_t stream);
 bool mfma_supported(int dtype, int head_dim, int block_m);
+// joins `splits` partial results (layout of AttnParams::part_o / part_lse) into o (and lse, may be null)
+int launch_merge_splits(const float* part_o, const float* part_lse, int splits, int64_t rows, int head_dim,
+                        void* o, int out_dtype, float* lse, hipStream_t stream);
 
 // ---- element conversion -------------------------------------------------
 __device__ __forceinline__ float to_float(float x) { return x; }

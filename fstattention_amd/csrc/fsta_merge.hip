@@ -49,6 +49,40 @@ __global__ __launch_bounds__(kMergeThreads) void merge_states_kernel(
     if (lse_out && chunk == 0) lse_out[row] = sum > 0.f ? m + log2f(sum) : -INFINITY;
 }
 
+// Joins the partial results of a key-split attention launch: `splits` normalised float32 rows
+// with their base-2 log-sum-exps per query row.  4 floats per lane and part.
+template <typename T>
+__global__ __launch_bounds__(kMergeThreads) void merge_splits_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_lse, int splits, int64_t rows,
+    int32_t chunks_per_row, T* __restrict__ o, float* __restrict__ lse) {
+    const int64_t idx = (int64_t)blockIdx.x * kMergeThreads + threadIdx.x;
+    const int64_t row = idx / chunks_per_row;
+    if (row >= rows) return;
+    const int chunk = (int)(idx - row * chunks_per_row);
+    float m = -INFINITY;
+    for (int s = 0; s < splits; ++s) m = fmaxf(m, part_lse[(size_t)s * rows + row]);
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    float sum = 0.f;
+    const size_t part_stride = (size_t)rows * chunks_per_row;   // in float4
+    const float4* src = reinterpret_cast<const float4*>(part_o) + (size_t)row * chunks_per_row + chunk;
+    for (int s = 0; s < splits; ++s) {
+        const float l = part_lse[(size_t)s * rows + row];
+        const float w = l == -INFINITY ? 0.f : exp2f(l - m);   // a part without keys drops out
+        const float4 x = src[(size_t)s * part_stride];
+        if (w > 0.f) {
+            acc[0] += w * x.x; acc[1] += w * x.y; acc[2] += w * x.z; acc[3] += w * x.w;
+            sum += w;
+        }
+    }
+    const float inv = sum > 0.f ? 1.f / sum : 0.f;
+    struct alignas(sizeof(T) * 4) Pack { T v[4]; };
+    Pack out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out.v[i] = from_float<T>(acc[i] * inv);
+    *reinterpret_cast<Pack*>(o + ((size_t)row * chunks_per_row + chunk) * 4) = out;
+    if (lse && chunk == 0) lse[row] = sum > 0.f ? m + log2f(sum) : -INFINITY;
+}
+
 template <typename T>
 int launch_merge(const void* o_a, const float* lse_a, const void* o_b, const float* lse_b, void* o_out,
                  float* lse_out, int64_t rows, int32_t head_dim, hipStream_t stream) {
@@ -64,6 +98,32 @@ int launch_merge(const void* o_a, const float* lse_a, const void* o_b, const flo
 }
 
 }  // namespace
+
+int launch_merge_splits(const float* part_o, const float* part_lse, int splits, int64_t rows, int head_dim,
+                        void* o, int out_dtype, float* lse, hipStream_t stream) {
+    const int chunks = head_dim / 4;
+    const int64_t blocks = (rows * chunks + kMergeThreads - 1) / kMergeThreads;
+    if (blocks > 0x7fffffff) return fail(FSTA_EUNSUPPORTED, "merge of key splits: %lld rows", (long long)rows);
+    const dim3 grid((unsigned)blocks), block(kMergeThreads);
+    switch (out_dtype) {
+        case FSTA_F32:
+            hipLaunchKernelGGL(merge_splits_kernel<float>, grid, block, 0, stream, part_o, part_lse, splits, rows,
+                               chunks, static_cast<float*>(o), lse);
+            break;
+        case FSTA_F16:
+            hipLaunchKernelGGL(merge_splits_kernel<__half>, grid, block, 0, stream, part_o, part_lse, splits, rows,
+                               chunks, static_cast<__half*>(o), lse);
+            break;
+        case FSTA_BF16:
+            hipLaunchKernelGGL(merge_splits_kernel<__hip_bfloat16>, grid, block, 0, stream, part_o, part_lse, splits,
+                               rows, chunks, static_cast<__hip_bfloat16*>(o), lse);
+            break;
+        default: return fail(FSTA_EINVAL, "merge of key splits: out_dtype=%d", out_dtype);
+    }
+    FSTA_HIP_OK(hipGetLastError());
+    return FSTA_OK;
+}
+
 }  // namespace fsta
 
 using namespace fsta;

@@ -14,6 +14,7 @@
 #ifndef FSTA_H
 #define FSTA_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -41,6 +42,11 @@ extern "C" {
 #define FSTA_FLAG_WIDE_WAVES 4u /* matrix-core kernel with 32 query rows per wave
                                   (32x32x16 MFMA, 2 waves per SIMD) instead of 16
                                   rows per wave (16x16x32 MFMA, 4 waves per SIMD) */
+
+#define FSTA_FLAG_KEY_SPLITS(n) (((uint32_t)(n) & 0xffu) << 8)
+                               /* fsta_attention_fwd_ws / fsta_attention_workspace_bytes:
+                                  cut the shared prefix into n runs of keys (n = 1: never
+                                  split; n = 0, i.e. no such flag: the library decides)   */
 
 /* bits of the status word written by fsta_precompute */
 #define FSTA_PRE_TOO_MANY_ANCESTORS 1u /* a block has more than max_ancestors unique ancestors */
@@ -118,6 +124,37 @@ int fsta_attention_fwd(const void* q, const void* k, const void* v, void* o, flo
                        int32_t dtype, int32_t out_dtype,
                        int32_t block_m, int32_t max_ancestors, int32_t num_blocks,
                        float sm_scale, uint32_t flags, void* stream);
+
+/*
+ * The same operation with a device workspace, which lets the library cut a long
+ * shared prefix (fstattention.py:113-136: every query block walks all nk - nq
+ * prefix keys on its own) into runs of keys that separate workgroups take
+ * ("flash decoding"): when batch * heads * num_blocks workgroups cannot fill
+ * the GPU, e.g. one sequence with a long KV cache in front of a small tree, the
+ * prefix is read several times faster.  Each run yields a float32 partial
+ * result with its log-sum-exp in the workspace; a second kernel joins them into
+ * o (and lse).  Results are those of fsta_attention_fwd up to float32 rounding
+ * of the join.
+ *   fsta_attention_workspace_bytes: bytes of device memory (256-byte aligned
+ *     start) fsta_attention_fwd_ws wants for this problem; 0 when it would not
+ *     split (short or no prefix, enough blocks, dtype/shape of the scalar kernel).
+ *   fsta_attention_fwd_ws: `workspace` of at least that many bytes, or NULL / a
+ *     smaller size to run without splitting (then identical to
+ *     fsta_attention_fwd).  The workspace is free again when the work queued on
+ *     `stream` has run; calls that share one workspace must not overlap.
+ * `flags` must be the same in both calls; FSTA_FLAG_KEY_SPLITS(n) forces n runs.
+ */
+size_t fsta_attention_workspace_bytes(int32_t batch, int32_t heads, int32_t nq, int32_t nk,
+                                      int32_t head_dim, int32_t dtype, int32_t block_m,
+                                      int32_t max_ancestors, float sm_scale, uint32_t flags);
+int fsta_attention_fwd_ws(const void* q, const void* k, const void* v, void* o, float* lse,
+                          const int64_t* ancestor_idx, const uint32_t* mask_bits,
+                          const int32_t* anc_count, const int64_t* leaf_idx,
+                          int32_t batch, int32_t heads, int32_t nq, int32_t nk, int32_t head_dim,
+                          int32_t dtype, int32_t out_dtype,
+                          int32_t block_m, int32_t max_ancestors, int32_t num_blocks,
+                          float sm_scale, uint32_t flags,
+                          void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * parent[n_nodes] int64 (parent[i] < i, -1 for roots) -> level_lookup [n_nodes]

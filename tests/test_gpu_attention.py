@@ -20,7 +20,7 @@ pytestmark = pytest.mark.gpu
 
 
 def run_tree(parent, block_m, z, h, d, dtype, seed, prefix=0, generic=False, fast_pv=False,
-             scale=None, check_lse=True, wide_waves=False):
+             scale=None, check_lse=True, wide_waves=False, key_splits=None):
     n = len(parent)
     a_idx, a_mask, l_idx, max_anc = oracle_inputs(parent, block_m)
     nb = a_idx.shape[0]
@@ -33,7 +33,7 @@ def run_tree(parent, block_m, z, h, d, dtype, seed, prefix=0, generic=False, fas
     o, lse = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(),
                            scale, BLOCK_M=block_m, MAX_ANCESTORS=max_anc,
                            out_dtype=torch.float32, return_lse=True, generic=generic, fast_pv=fast_pv,
-                           wide_waves=wide_waves)
+                           wide_waves=wide_waves, key_splits=key_splits)
     assert o.dtype == torch.float32 and o.shape == q.shape
     err = assert_close(o, want, dtype, f"n={n} m={block_m} d={d} {dtype} prefix={prefix}")
     if check_lse:
@@ -95,6 +95,63 @@ def test_shapes_sweep_wide_wave_variant(dtype, d, block_m, prefix):
 def test_shared_prefix(dtype, prefix):
     parent = trees.random_recursive_parents(128, 5, window=32)
     run_tree(parent, 64, 2, 2, 64, dtype, 11, prefix=prefix)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("block_m,d", [(32, 64), (64, 128), (128, 128), (64, 32)])
+@pytest.mark.parametrize("prefix,splits", [(300, 3), (1024, 4), (77, 2), (2048, None), (96, 3)])
+def test_prefix_cut_into_key_runs(dtype, block_m, d, prefix, splits):
+    """The shared prefix taken by several workgroups per block (forced counts, and the library's
+    own choice for a long prefix in front of few blocks) against the oracle over all keys."""
+    parent = trees.random_recursive_parents(200, 300 + d + block_m, window=48)
+    run_tree(parent, block_m, 1, 3, d, dtype, 13, prefix=prefix, key_splits=splits)
+
+
+def test_key_runs_native_output_type_and_workspace_contract():
+    """Output in the storage type through the joining kernel; the C entry point with no or too
+    small a workspace runs unsplit; the workspace query is 0 where no split is planned."""
+    from fstattention_amd import _lib
+    from fstattention_amd.attention import _DTYPES, _packed_for
+    lib = _lib.load()
+    cfg = trees.config(2)
+    prefix, m, d, h = 4096, cfg.block_m, cfg.head_dim, 4
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(cfg.parent, m)
+    nq = a_idx.shape[0] * m
+    q, k, v = rand_qkv(1, h, nq, nq + prefix, d, torch.bfloat16, 21)
+    scale = 1.0 / math.sqrt(d)
+    want, want_lse = dense_oracle(q, k, v, cfg.parent, scale, prefix=prefix, nq_pad=nq - len(cfg.parent))
+    a_idx, l_idx = shift_for_prefix(a_idx, l_idx, prefix)
+    qd, kd, vd, ad, md, ld = (t.cuda() for t in (q, k, v, a_idx, a_mask, l_idx))
+    o, lse = fst_attention(qd, kd, vd, ad, md, ld, scale, BLOCK_M=m, MAX_ANCESTORS=max_anc, return_lse=True)
+    assert o.dtype == torch.bfloat16
+    # one rounding to bfloat16 on top of the float32 tolerance
+    torch.testing.assert_close(o.cpu().double(), want, atol=2e-3 + 2 ** -8, rtol=2e-3 + 2 ** -8)
+    torch.testing.assert_close(lse.cpu().double().view(1, h, nq), want_lse, atol=2e-3, rtol=2e-3)
+
+    code = _DTYPES[torch.bfloat16]
+    need = lib.fsta_attention_workspace_bytes(1, h, nq, nq + prefix, d, code, m, max_anc, scale, 0)
+    assert need > 0
+    assert lib.fsta_attention_workspace_bytes(1, h, nq, nq, d, code, m, max_anc, scale, 0) == 0
+    assert lib.fsta_attention_workspace_bytes(1, h, nq, nq + prefix, d, code, m, max_anc, scale,
+                                              _lib.flag_key_splits(1)) == 0
+    assert lib.fsta_attention_workspace_bytes(1, h, nq, nq + prefix, d, _DTYPES[torch.float32], m, max_anc,
+                                              scale, 0) == 0
+    packed = _packed_for(ad, md)
+    outs = []
+    for work_bytes in (0, need - 1, need):
+        work = torch.empty((max(work_bytes, 1),), dtype=torch.uint8, device="cuda")
+        o32 = torch.empty(q.shape, dtype=torch.float32, device="cuda")
+        _lib.check(lib.fsta_attention_fwd_ws(
+            qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o32.data_ptr(), None, ad.data_ptr(),
+            packed.mask_bits.data_ptr(), packed.anc_count.data_ptr(), ld.data_ptr(), 1, h, nq, nq + prefix, d,
+            code, _DTYPES[torch.float32], m, max_anc, a_idx.shape[0], scale, 0,
+            work.data_ptr() if work_bytes else None, work_bytes, torch.cuda.current_stream().cuda_stream))
+        assert_close(o32, want, torch.bfloat16, f"workspace of {work_bytes} bytes")
+        outs.append(o32)
+    unsplit = fst_attention(qd, kd, vd, ad, md, ld, scale, BLOCK_M=m, MAX_ANCESTORS=max_anc,
+                            out_dtype=torch.float32, key_splits=1)
+    assert torch.equal(outs[0], unsplit) and torch.equal(outs[1], unsplit)
+    assert not torch.equal(outs[2], unsplit)      # the split path did run
 
 
 def test_reference_test_shape_with_and_without_prefix():
