@@ -79,6 +79,39 @@ def test_argument_validation_happens_before_any_gpu_work():
         _lib.check(_lib.EINVAL)
 
 
+def test_workspace_planning_is_host_arithmetic():
+    """How a shared prefix is cut into runs of keys depends on the shape and flags only."""
+    lib = _lib.load()
+    per_run = 32 * 256 * (128 + 1) * 4       # float32 partial rows + their log-sum-exps of one run
+    size = lambda *a: lib.fsta_attention_workspace_bytes(*a)
+    # one sequence, 32 heads, 4 blocks of 64 rows behind 16384 prefix keys: 128 workgroups -> 4 runs
+    assert size(1, 32, 256, 256 + 16384, 128, _lib.BF16, 64, 64, 0.1, 0) == 4 * per_run
+    assert size(1, 32, 256, 256 + 16384, 128, _lib.BF16, 64, 64, 0.1, _lib.flag_key_splits(7)) == 7 * per_run
+    # nothing to cut: no prefix, a short one, enough blocks already, never-split flag
+    assert size(1, 32, 256, 256, 128, _lib.BF16, 64, 64, 0.1, 0) == 0
+    assert size(1, 32, 256, 256 + 256, 128, _lib.BF16, 64, 64, 0.1, 0) == 0
+    assert size(8, 32, 256, 256 + 16384, 128, _lib.BF16, 64, 64, 0.1, 0) == 0
+    assert size(1, 32, 256, 256 + 16384, 128, _lib.BF16, 64, 64, 0.1, _lib.flag_key_splits(1)) == 0
+    # kernels without key runs: float32, the scalar and wide-wave kernels, non-positive scales
+    assert size(1, 32, 256, 256 + 16384, 128, _lib.F32, 64, 64, 0.1, 0) == 0
+    assert size(1, 32, 256, 256 + 16384, 128, _lib.BF16, 64, 64, 0.1, _lib.FLAG_GENERIC) == 0
+    assert size(1, 32, 256, 256 + 16384, 128, _lib.BF16, 64, 64, 0.1, _lib.FLAG_WIDE_WAVES) == 0
+    assert size(1, 32, 256, 256 + 16384, 128, _lib.BF16, 64, 64, 0.0, 0) == 0
+    assert size(1, 32, 256, 256 + 16384, 128, _lib.BF16, 16, 64, 0.1, 0) == 0
+    # more runs than tiles are not made; malformed shapes want nothing
+    assert size(1, 1, 32, 32 + 64, 64, _lib.F16, 32, 16, 0.1, _lib.flag_key_splits(9)) == 2 * 32 * (64 + 1) * 4
+    assert size(0, 32, 256, 512, 128, _lib.BF16, 64, 64, 0.1, 0) == 0
+    assert size(1, 32, 256, 100, 128, _lib.BF16, 64, 64, 0.1, 0) == 0
+    # the workspace variant validates like the plain one, and wants an aligned workspace
+    bad = lib.fsta_attention_fwd_ws(None, None, None, None, None, None, None, None, None,
+                                    1, 1, 16, 16, 64, 7, 7, 16, 8, 1, 1.0, 0, None, 0, None)
+    assert bad == _lib.EINVAL and b"dtype" in lib.fsta_last_error()
+    need = size(1, 32, 256, 256 + 16384, 128, _lib.BF16, 64, 64, 0.1, 0)
+    odd = lib.fsta_attention_fwd_ws(8, 8, 8, 8, None, 8, 8, None, 8, 1, 32, 256, 256 + 16384, 128, _lib.BF16,
+                                    _lib.BF16, 64, 64, 4, 0.1, 0, 4100, need, None)
+    assert odd == _lib.EINVAL and b"aligned" in lib.fsta_last_error()
+
+
 def test_python_entry_points_refuse_to_run_without_a_gpu_path():
     import torch
     from fstattention_amd import create_fst_attention_kernel_inputs, fst_attention, trees
