@@ -10,15 +10,20 @@ namespace {
 
 constexpr int kThreads = 256;
 
-// Dynamic LDS of block_precompute_kernel:
-//   bitmap[W] | rank_base[W] | mbits[mask_words * M] | lvl[M] | partial[kThreads] | misc[4]
+constexpr int kMaxThreads = 1024;   // block_precompute_kernel runs with 256 or 1024 threads
+constexpr int kBatch = 8;           // independent loads a thread has in flight
+
+// Dynamic LDS of block_precompute_kernel (32-bit words):
+//   bitmap[W] | rank_base[W] | mbits[mask_words * M] | lvl[M] | misc[4] | vals[staged]
+// vals: the block's lineage rows as int32 (when they fit), so that the second pass over them
+// reads LDS instead of going to memory again.
 __host__ __device__ inline size_t precompute_lds_words(int64_t n_words, int mask_words, int block_m) {
-    return (size_t)(2 * n_words) + (size_t)mask_words * block_m + block_m + kThreads + 4;
+    return (size_t)(2 * n_words) + (size_t)mask_words * block_m + block_m + 4;
 }
 
-__global__ __launch_bounds__(kThreads) void block_precompute_kernel(
+__global__ __launch_bounds__(kMaxThreads) void block_precompute_kernel(
     int64_t* __restrict__ lineage, const int64_t* __restrict__ level_lookup,
-    int64_t n_nodes, int64_t width, int block_m, int max_anc, int mask_words, int mutate,
+    int64_t n_nodes, int64_t width, int block_m, int max_anc, int mask_words, int mutate, int staged,
     int64_t* __restrict__ ancestor_idx, uint8_t* __restrict__ ancestor_mask,
     int64_t* __restrict__ leaf_idx, uint32_t* __restrict__ mask_bits,
     int32_t* __restrict__ anc_count, uint32_t* __restrict__ status) {
@@ -28,19 +33,34 @@ __global__ __launch_bounds__(kThreads) void block_precompute_kernel(
     uint32_t* rank_base = bitmap + n_words;                   // set bits in lower words
     uint32_t* mbits = rank_base + n_words;                    // [mask_words][block_m]
     int32_t* lvl_s = reinterpret_cast<int32_t*>(mbits + (size_t)mask_words * block_m);  // [block_m]
-    uint32_t* partial = reinterpret_cast<uint32_t*>(lvl_s + block_m);                   // [kThreads]
-    uint32_t* misc = partial + kThreads;  // [0] a -1 was seen, [1] error bits, [2] total count
+    uint32_t* misc = reinterpret_cast<uint32_t*>(lvl_s + block_m);   // [0] a -1 was seen, [2] total count
+    int32_t* vals_s = reinterpret_cast<int32_t*>(misc + 4);          // [rows * width] when staged
 
     const int tid = threadIdx.x;
+    const int threads = blockDim.x;
     const int j = blockIdx.x;
     const int64_t lo = (int64_t)j * block_m;
     const int rows = (int)min((int64_t)block_m, n_nodes - lo);
 
-    for (int w = tid; w < n_words; w += kThreads) bitmap[w] = 0u;
-    for (int e = tid; e < mask_words * block_m; e += kThreads) mbits[e] = 0u;
+    // The first kBatch lineage entries of every thread are requested before anything else; they
+    // are on their way while the LDS tables are cleared.
+    const int64_t* chunk = lineage + lo * width;
+    const uint32_t n_elem = (uint32_t)rows * (uint32_t)width;   // the host checked that this fits
+    auto load_batch = [&](uint32_t e0, int64_t (&val)[kBatch]) {
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {
+            const uint32_t e = e0 + (uint32_t)b * threads;
+            val[b] = e < n_elem ? chunk[e] : 0;
+        }
+    };
+    int64_t first[kBatch];
+    load_batch(tid, first);
+
+    for (int w = tid; w < n_words; w += threads) bitmap[w] = 0u;
+    for (int e = tid; e < mask_words * block_m; e += threads) mbits[e] = 0u;
     if (tid < 4) misc[tid] = 0u;
     uint32_t err = 0u;
-    for (int r = tid; r < block_m; r += kThreads) {
+    for (int r = tid; r < block_m; r += threads) {
         int32_t lv = -1;  // -1 = nothing to insert (pad row or invalid level)
         if (r < rows) {
             int64_t l = level_lookup[lo + r];
@@ -52,46 +72,62 @@ __global__ __launch_bounds__(kThreads) void block_precompute_kernel(
     }
     __syncthreads();
 
-    // 1. set a bit for every value of the block's lineage rows (utils.py:118-119)
-    const int64_t* chunk = lineage + lo * width;
-    const int64_t n_elem = (int64_t)rows * width;
+    // 1. set a bit for every value of the block's lineage rows (utils.py:118-119); kBatch loads
+    //    per thread go out before the first one is used
     bool saw_pad = false;
-    for (int64_t e = tid; e < n_elem; e += kThreads) {
-        const int64_t val = chunk[e];
-        if (val == -1) saw_pad = true;
-        else if (val < -1 || val >= n_nodes) err |= FSTA_PRE_BAD_NODE_ID;
-        else atomicOr(&bitmap[val >> 5], 1u << (val & 31));
+    auto take_batch = [&](uint32_t e0, const int64_t (&val)[kBatch]) {
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {
+            const uint32_t e = e0 + (uint32_t)b * threads;
+            if (e >= n_elem) break;
+            int32_t keep = -1;
+            if (val[b] == -1) saw_pad = true;
+            else if (val[b] < -1 || val[b] >= n_nodes) err |= FSTA_PRE_BAD_NODE_ID;
+            else {
+                // rows of one block share most of their ancestors: only a bit that is not there
+                // yet goes through the (serialising) atomic
+                keep = (int32_t)val[b];
+                const uint32_t bit = 1u << (keep & 31);
+                if (!(bitmap[keep >> 5] & bit)) atomicOr(&bitmap[keep >> 5], bit);
+            }
+            if (staged) vals_s[e] = keep;
+        }
+    };
+    take_batch(tid, first);
+    for (uint32_t e0 = tid + (uint32_t)threads * kBatch; e0 < n_elem; e0 += (uint32_t)threads * kBatch) {
+        int64_t val[kBatch];
+        load_batch(e0, val);
+        take_batch(e0, val);
     }
     if (saw_pad) misc[0] = 1u;
     __syncthreads();
 
-    // The reference drops the smallest unique value unconditionally (utils.py:119,
-    // the `[1:]`); that is the -1 padding whenever one is present.  Without any
-    // -1 in the block the smallest node id goes instead.
-    if (tid == 0 && misc[0] == 0u) {
-        for (int w = 0; w < n_words; ++w) {
-            if (bitmap[w]) { bitmap[w] &= bitmap[w] - 1u; break; }
+    // 2. exclusive prefix sum of the per-word popcounts -> rank of every ancestor; the first
+    //    wave scans, each lane a run of consecutive words
+    if (tid < 64) {
+        // The reference drops the smallest unique value unconditionally (utils.py:119, the
+        // `[1:]`); that is the -1 padding whenever one is present.  Without any -1 in the block
+        // the smallest node id goes instead.  (Same wave as the scan: its LDS accesses stay in order.)
+        if (tid == 0 && misc[0] == 0u) {
+            for (int w = 0; w < n_words; ++w) {
+                if (bitmap[w]) { bitmap[w] &= bitmap[w] - 1u; break; }
+            }
         }
-    }
-    __syncthreads();
-
-    // 2. exclusive prefix sum of the per-word popcounts -> rank of every ancestor
-    const int per_thread = (n_words + kThreads - 1) / kThreads;
-    const int w_begin = min(tid * per_thread, n_words);
-    const int w_end = min(w_begin + per_thread, n_words);
-    uint32_t local = 0u;
-    for (int w = w_begin; w < w_end; ++w) local += __popc(bitmap[w]);
-    partial[tid] = local;
-    __syncthreads();
-    if (tid == 0) {
-        uint32_t run = 0u;
-        for (int t = 0; t < kThreads; ++t) { const uint32_t c = partial[t]; partial[t] = run; run += c; }
-        misc[2] = run;
-    }
-    __syncthreads();
-    {
-        uint32_t run = partial[tid];
+        __builtin_amdgcn_wave_barrier();
+        const int per_lane = (n_words + 63) / 64;
+        const int w_begin = min(tid * per_lane, n_words);
+        const int w_end = min(w_begin + per_lane, n_words);
+        uint32_t local = 0u;
+        for (int w = w_begin; w < w_end; ++w) local += __popc(bitmap[w]);
+        uint32_t incl = local;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t up = __shfl_up(incl, d, 64);
+            if (tid >= d) incl += up;
+        }
+        uint32_t run = incl - local;
         for (int w = w_begin; w < w_end; ++w) { rank_base[w] = run; run += __popc(bitmap[w]); }
+        if (tid == 63) misc[2] = incl;
     }
     __syncthreads();
     const uint32_t total = misc[2];
@@ -99,8 +135,8 @@ __global__ __launch_bounds__(kThreads) void block_precompute_kernel(
     const int kept = (int)min(total, (uint32_t)max_anc);
 
     // 3. ancestor_idx: ascending ids, left aligned, -1 padded (utils.py:112,120)
-    for (int c = kept + tid; c < max_anc; c += kThreads) ancestor_idx[(size_t)j * max_anc + c] = -1;
-    for (int w = tid; w < n_words; w += kThreads) {
+    for (int c = kept + tid; c < max_anc; c += threads) ancestor_idx[(size_t)j * max_anc + c] = -1;
+    for (int w = tid; w < n_words; w += threads) {
         uint32_t bits = bitmap[w];
         uint32_t r = rank_base[w];
         while (bits) {
@@ -114,7 +150,7 @@ __global__ __launch_bounds__(kThreads) void block_precompute_kernel(
 
     // 4. leaves: ids of the block's range that are not in the set; the range is
     //    not clipped to n_nodes (utils.py:121-122)
-    for (int r = tid; r < block_m; r += kThreads) {
+    for (int r = tid; r < block_m; r += threads) {
         const int64_t id = lo + r;
         const bool is_anc = id < n_nodes && ((bitmap[id >> 5] >> (id & 31)) & 1u);
         leaf_idx[(size_t)j * block_m + r] = is_anc ? -1 : id;
@@ -122,35 +158,70 @@ __global__ __launch_bounds__(kThreads) void block_precompute_kernel(
 
     // 5. mask: row r holds its lineage plus itself in its own level column
     //    (utils.py:124-127); membership of ancestor c in that row
-    for (int64_t e = tid; e < n_elem; e += kThreads) {
-        const int r = (int)(e / width);
-        const int l = (int)(e - (int64_t)r * width);
-        const int64_t val = (l == lvl_s[r]) ? lo + r : chunk[e];
-        if (val < 0 || val >= n_nodes) continue;
-        const uint32_t word = bitmap[val >> 5];
-        const uint32_t bit = 1u << (val & 31);
-        if (!(word & bit)) continue;
-        const uint32_t rank = rank_base[val >> 5] + __popc(word & (bit - 1u));
-        if (rank < (uint32_t)max_anc) atomicOr(&mbits[(rank >> 5) * block_m + r], 1u << (rank & 31));
+    //    A thread walks a run of consecutive levels of one row.  Ancestors along a path have
+    //    increasing ids, hence increasing ranks: the bits of a run fall into one or two mask words,
+    //    which are collected in a register and merged with one atomic each.
+    {
+        const int segs_per_row = max(1, min((int)width, threads / max(rows, 1)));
+        const int seg_len = ((int)width + segs_per_row - 1) / segs_per_row;
+        for (int sidx = tid; sidx < rows * segs_per_row; sidx += threads) {
+            const int r = sidx / segs_per_row;
+            const int l0 = (sidx - r * segs_per_row) * seg_len;
+            const int l1 = min(l0 + seg_len, (int)width);
+            const int own = lvl_s[r];
+            const uint32_t base = (uint32_t)r * (uint32_t)width;
+            uint32_t cur = 0xffffffffu, acc = 0u;
+            for (int l = l0; l < l1; ++l) {
+                const int64_t val = l == own ? lo + r : (staged ? (int64_t)vals_s[base + l] : chunk[base + l]);
+                if (val < 0 || val >= n_nodes) continue;
+                const uint32_t word = bitmap[val >> 5];
+                const uint32_t bit = 1u << (val & 31);
+                if (!(word & bit)) continue;
+                const uint32_t rank = rank_base[val >> 5] + __popc(word & (bit - 1u));
+                if (rank >= (uint32_t)max_anc) continue;
+                if ((rank >> 5) != cur) {
+                    if (acc) atomicOr(&mbits[cur * block_m + r], acc);
+                    cur = rank >> 5;
+                    acc = 0u;
+                }
+                acc |= 1u << (rank & 31);
+            }
+            if (acc) atomicOr(&mbits[cur * block_m + r], acc);
+        }
     }
     __syncthreads();
 
     if (mask_bits) {
-        for (int e = tid; e < mask_words * block_m; e += kThreads)
+        for (int e = tid; e < mask_words * block_m; e += threads)
             mask_bits[(size_t)j * mask_words * block_m + e] = mbits[e];
     }
     if (ancestor_mask) {
+        // one byte per (row, ancestor slot); 8 slots of a row per store where the layout allows
         uint8_t* out = ancestor_mask + (size_t)j * block_m * max_anc;
-        const int n_out = block_m * max_anc;
-        for (int e = tid; e < n_out; e += kThreads) {
-            const int r = e / max_anc, c = e - r * max_anc;
-            out[e] = (uint8_t)((mbits[(c >> 5) * block_m + r] >> (c & 31)) & 1u);
+        if (max_anc % 8 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0) {
+            const int per_row = max_anc / 8;
+            for (int e = tid; e < block_m * per_row; e += threads) {
+                const int r = e / per_row, c = (e - r * per_row) * 8;
+                const uint32_t bits = (mbits[(c >> 5) * block_m + r] >> (c & 31)) & 0xffu;
+                // bit i -> byte i: three doubling steps spread the 8 bits over 64
+                uint64_t x = bits;
+                x = (x | (x << 28)) & 0x0000000f0000000full;
+                x = (x | (x << 14)) & 0x0003000300030003ull;
+                x = (x | (x << 7)) & 0x0101010101010101ull;
+                reinterpret_cast<uint64_t*>(out)[e] = x;
+            }
+        } else {
+            const int n_out = block_m * max_anc;
+            for (int e = tid; e < n_out; e += threads) {
+                const int r = e / max_anc, c = e - r * max_anc;
+                out[e] = (uint8_t)((mbits[(c >> 5) * block_m + r] >> (c & 31)) & 1u);
+            }
         }
     }
 
     // 6. the caller's lineage receives the self entries (utils.py:118,125)
     if (mutate) {
-        for (int r = tid; r < rows; r += kThreads)
+        for (int r = tid; r < rows; r += threads)
             if (lvl_s[r] >= 0) lineage[(lo + r) * width + lvl_s[r]] = lo + r;
     }
     if (err) atomicOr(status, err);
@@ -254,19 +325,28 @@ extern "C" int fsta_precompute(int64_t* lineage, const int64_t* level_lookup, in
     if (block_m > 4096) return fail(FSTA_EUNSUPPORTED, "fsta_precompute: block_m=%d > 4096", block_m);
     const int mask_words = fsta_mask_words(max_ancestors);
     const int64_t n_words = (n_nodes + 31) >> 5;
-    const size_t lds = sizeof(uint32_t) * precompute_lds_words(n_words, mask_words, block_m);
+    if ((int64_t)block_m * width > 0x7fffffff)
+        return fail(FSTA_EUNSUPPORTED, "fsta_precompute: block_m=%d x width=%lld entries per block", block_m,
+                    (long long)width);
+    size_t lds = sizeof(uint32_t) * precompute_lds_words(n_words, mask_words, block_m);
     if (lds > 160 * 1024)
         return fail(FSTA_EUNSUPPORTED,
                     "fsta_precompute: n_nodes=%lld block_m=%d max_ancestors=%d need %zu bytes of LDS (limit 163840)",
                     (long long)n_nodes, block_m, max_ancestors, lds);
+    // the block's lineage rows stay in LDS between the two passes over them when they fit
+    const size_t entries = (size_t)block_m * (size_t)width;
+    const int staged = lds + entries * 4 <= 160 * 1024 ? 1 : 0;
+    if (staged) lds += entries * 4;
     if (lds > 64 * 1024) {
         const int rc = allow_full_lds<&block_precompute_kernel>();
         if (rc != FSTA_OK) return rc;
     }
     const int64_t nb = (n_nodes + block_m - 1) / block_m;
-    hipLaunchKernelGGL(block_precompute_kernel, dim3((unsigned)nb), dim3(kThreads), lds,
+    // a block with many entries is worked on by 16 waves, else by 4
+    const int threads = entries >= 2048 || (size_t)block_m * max_ancestors >= 8192 ? kMaxThreads : kThreads;
+    hipLaunchKernelGGL(block_precompute_kernel, dim3((unsigned)nb), dim3(threads), lds,
                        static_cast<hipStream_t>(stream), lineage, level_lookup, n_nodes, width,
-                       block_m, max_ancestors, mask_words, mutate_lineage, ancestor_idx,
+                       block_m, max_ancestors, mask_words, mutate_lineage, staged, ancestor_idx,
                        ancestor_mask, leaf_idx, mask_bits, anc_count, status);
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
