@@ -46,7 +46,7 @@ int fail(int code, const char* fmt, ...);
             return ::fsta::fail(FSTA_EHIP, "%s: %s", #expr, hipGetErrorString(err__)); \
     } while (0)
 
-// Raises the dynamic-LDS limit of one kernel to the 160 KB of a gfx950 CU, once per device and
+// Raises the dynamic-LDS limit of one kernel to what the 160 KB of a gfx950 CU leave, once per device and
 // process (the attribute call costs microseconds on the host; setting it twice in a race is harmless).
 template <auto Kernel>
 int allow_full_lds() {
@@ -55,8 +55,11 @@ int allow_full_lds() {
     FSTA_HIP_OK(hipGetDevice(&dev));
     const bool tracked = dev >= 0 && dev < 64;
     if (tracked && done[dev]) return FSTA_OK;
+    // static LDS of the kernel (its own or a library routine's) counts against the same 160 KB
+    hipFuncAttributes attr;
+    FSTA_HIP_OK(hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(Kernel)));
     FSTA_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    160 * 1024));
+                                    160 * 1024 - (int)attr.sharedSizeBytes));
     if (tracked) done[dev] = true;
     return FSTA_OK;
 }

@@ -123,6 +123,102 @@ __global__ __launch_bounds__(kOrderThreads) void order_finish_kernel(const int64
     rank[i] = pre;
 }
 
+// Trees of a few thousand nodes (what speculative decoding builds) in ONE workgroup and launch:
+// the four steps above with every array in LDS, so that a hop or a sibling visit is an LDS
+// access and the steps are separated by barriers instead of kernel boundaries.  Siblings are
+// found through per-parent child lists (built with atomic exchanges) instead of the all-pairs
+// loop: a node visits its parent's other children only.  A list is a chain of dependent reads,
+// so children of a parent with more than kListedChildren of them (no tree of speculative decoding
+// has such nodes) scan the whole node array instead, whose reads are independent.
+// (Tried and dropped: path sums by pointer doubling and sizes level by level.  Fewer dependent
+// hops, but every round ends in a barrier of 16 waves, which costs more than the hops it saves
+// on trees up to 160 levels deep.)
+constexpr int kSmallThreads = 1024;
+constexpr int kSmallMaxNodes = 4096;   // 6 int32 arrays of n (+1) entries: 96 KB of LDS
+constexpr int kListedChildren = 64;
+
+__global__ __launch_bounds__(kSmallThreads) void order_small_kernel(const int64_t* __restrict__ parent, int n,
+                                                                    int light_first, int64_t* __restrict__ perm,
+                                                                    int64_t* __restrict__ rank,
+                                                                    uint32_t* __restrict__ status) {
+    extern __shared__ int32_t small_s[];
+    int32_t* par_s = small_s;          // [n]   parent, -1 for roots
+    int32_t* size_s = par_s + n;       // [n]   nodes in the subtree
+    int32_t* off_s = size_s + n;       // [n]   sizes of the siblings visited earlier
+    int32_t* next_s = off_s + n;       // [n]   next child of the same parent
+    int32_t* head_s = next_s + n;      // [n+1] first child; entry n: the roots
+    int32_t* kids_s = head_s + n + 1;  // [n+1] number of children
+    int32_t* bad_s = kids_s + n + 1;   // [1]   malformed input
+    const int tid = threadIdx.x;
+    if (tid == 0) *bad_s = 0;
+    for (int i = tid; i <= n; i += kSmallThreads) {
+        head_s[i] = -1;
+        kids_s[i] = 0;
+    }
+    __syncthreads();
+    for (int i = tid; i < n; i += kSmallThreads) {
+        const int64_t p = parent[i];
+        const bool ok = p >= -1 && p < i;     // every hop goes to a smaller id: the walks end
+        par_s[i] = ok ? (int32_t)p : -1;
+        size_s[i] = 1;
+        if (!ok) *bad_s = 1;
+    }
+    __syncthreads();
+    if (*bad_s) {      // malformed parent array: identity, the caller reads the status word
+        for (int i = tid; i < n; i += kSmallThreads) {
+            perm[i] = i;
+            rank[i] = i;
+        }
+        if (tid == 0) atomicOr(status, FSTA_PRE_BAD_NODE_ID);
+        return;
+    }
+    for (int i = tid; i < n; i += kSmallThreads) {
+        const int32_t p = par_s[i];
+        next_s[i] = atomicExch(&head_s[p >= 0 ? p : n], i);
+        atomicAdd(&kids_s[p >= 0 ? p : n], 1);
+        // Every node adds 1 to each of its ancestors.  Nodes with neighbouring ids meet after a
+        // few hops: where all lanes of the wave that are still walking stand on the same node,
+        // one of them adds for all (otherwise the adds of a shallow tree queue up at its root).
+        for (int32_t a = p; a >= 0; a = par_s[a]) {
+            const uint64_t walking = __ballot(true);
+            const int32_t first = __builtin_amdgcn_readfirstlane(a);
+            if (__ballot(a != first) == 0ull) {
+                if ((tid & 63) == __ffsll((long long)walking) - 1) atomicAdd(&size_s[first], __popcll(walking));
+            } else {
+                atomicAdd(&size_s[a], 1);
+            }
+        }
+    }
+    __syncthreads();
+    for (int i = tid; i < n; i += kSmallThreads) {
+        const int32_t p = par_s[i];
+        const int32_t my_key = light_first ? (size_s[i] << 13) | i : i;    // sizes and ids are below 2^13
+        int32_t acc = 0;
+        if (kids_s[p >= 0 ? p : n] <= kListedChildren) {
+            for (int32_t s = head_s[p >= 0 ? p : n]; s >= 0; s = next_s[s]) {
+                const int32_t sz = size_s[s];
+                const int32_t key = light_first ? (sz << 13) | s : s;
+                acc += key < my_key ? sz : 0;
+            }
+        } else {
+#pragma unroll 4
+            for (int32_t s = 0; s < n; ++s) {
+                const int32_t sz = size_s[s];
+                const int32_t key = light_first ? (sz << 13) | s : s;
+                acc += (par_s[s] == p && key < my_key) ? sz : 0;
+            }
+        }
+        off_s[i] = acc;
+    }
+    __syncthreads();
+    for (int i = tid; i < n; i += kSmallThreads) {
+        int32_t pre = -1;
+        for (int32_t cur = i; cur >= 0; cur = par_s[cur]) pre += off_s[cur] + 1;
+        perm[pre] = i;
+        rank[i] = pre;
+    }
+}
+
 }  // namespace
 }  // namespace fsta
 
@@ -138,6 +234,17 @@ extern "C" int fsta_dfs_order(const int64_t* parent, int64_t n_nodes, int32_t li
     if (!parent || !perm || !rank || !workspace || !status)
         return fail(FSTA_EINVAL, "fsta_dfs_order: null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (n_nodes <= kSmallMaxNodes) {
+        const size_t lds = (size_t)(6 * n_nodes + 3) * sizeof(int32_t);
+        if (lds > 64 * 1024) {
+            const int rc = allow_full_lds<&order_small_kernel>();
+            if (rc != FSTA_OK) return rc;
+        }
+        hipLaunchKernelGGL(order_small_kernel, dim3(1), dim3(kSmallThreads), lds, s, parent, (int)n_nodes,
+                           light_first ? 1 : 0, perm, rank, status);
+        FSTA_HIP_OK(hipGetLastError());
+        return FSTA_OK;
+    }
     int32_t* size = workspace;
     int32_t* off = workspace + n_nodes;
     const unsigned blocks = (unsigned)((n_nodes + kOrderThreads - 1) / kOrderThreads);

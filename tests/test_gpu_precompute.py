@@ -149,11 +149,18 @@ def test_lineage_from_parents_on_gpu():
 @pytest.mark.parametrize("children", ["index", "light_first"])
 def test_dfs_order_on_gpu_matches_the_host_order(children):
     cases = [np.array([-1], dtype=np.int64), np.array([-1, -1, -1], dtype=np.int64)]
-    for seed, n, window in [(1, 2, None), (2, 300, None), (3, 1500, 8), (4, 2049, 64)]:
+    # up to 4096 nodes one workgroup does everything, beyond that four launches do
+    for seed, n, window in [(1, 2, None), (2, 300, None), (3, 1500, 8), (4, 2049, 64), (5, 4096, 200),
+                            (6, 4097, 16), (7, 9000, None)]:
         parent = trees.random_recursive_parents(n, seed, window)
         parent[::101] = -1                      # forest
         cases.append(parent)
     cases += [trees.config(i).parent for i in (2, 3, 4, 5)]
+    star = np.zeros(700, dtype=np.int64)        # one parent with more children than a child list is walked for
+    star[0] = -1
+    star[500:] = np.arange(300, 500)            # ... and a second generation below some of them
+    cases.append(star)
+    cases.append(np.full(100, -1, dtype=np.int64))   # 100 roots
     for parent in cases:
         want = trees.dfs_order(parent, children)
         dev_parent = torch.from_numpy(parent).cuda()
