@@ -304,6 +304,52 @@ __global__ __launch_bounds__(kThreads) void lineage_from_parents_kernel(
     if (err) atomicOr(status, err);
 }
 
+// The same result for trees whose parent array and a piece of the output fit into LDS: a
+// workgroup owns `rows_per_wg` consecutive nodes.  One lane per node walks to the root ONCE,
+// noting the ancestors in hop order in an LDS row; the depth is the hop count.  Then all lanes
+// write the rows out, reversed into level order and padded with -1, as whole 512-byte pieces
+// (the walk above stores 8 bytes per lane into 64 different rows per instruction).
+__global__ __launch_bounds__(kThreads) void lineage_rows_kernel(
+    const int64_t* __restrict__ parent, int n, int width, int rows_per_wg,
+    int64_t* __restrict__ lineage, int64_t* __restrict__ level_lookup, uint32_t* __restrict__ status) {
+    extern __shared__ int32_t rows_s[];
+    int32_t* par_s = rows_s;                  // [n]
+    int32_t* depth_s = par_s + n;             // [rows_per_wg], -1: the row stays empty
+    int32_t* hops_s = depth_s + rows_per_wg;  // [rows_per_wg][width] ancestors, nearest first
+    const int tid = threadIdx.x;
+    for (int x = tid; x < n; x += kThreads) {
+        const int64_t v = parent[x];
+        par_s[x] = (v >= -1 && v < x) ? (int32_t)v : -2;   // -2: malformed entry
+    }
+    __syncthreads();
+    const int first = blockIdx.x * rows_per_wg;
+    const int rows = min(rows_per_wg, n - first);
+    uint32_t err = 0u;
+    for (int t = tid; t < rows; t += kThreads) {
+        int32_t* mine = hops_s + (size_t)t * width;
+        int hops = 0;
+        int32_t a = par_s[first + t];
+        for (; a >= 0; a = par_s[a]) {        // every hop goes to a smaller id, so the walk ends
+            if (hops < width) mine[hops] = a;
+            ++hops;
+        }
+        if (a < -1) err |= FSTA_PRE_BAD_NODE_ID;
+        else if (hops >= width) err |= FSTA_PRE_BAD_LEVEL;
+        level_lookup[first + t] = hops;
+        depth_s[t] = (a < -1 || hops >= width) ? -1 : hops;
+    }
+    __syncthreads();
+    int64_t* out = lineage + (size_t)first * width;
+    const uint32_t n_out = (uint32_t)rows * (uint32_t)width;
+    for (uint32_t e = tid; e < n_out; e += kThreads) {
+        const uint32_t t = e / (uint32_t)width;
+        const int l = (int)(e - t * (uint32_t)width);
+        const int d = depth_s[t];
+        out[e] = l < d ? (int64_t)hops_s[(size_t)t * width + (d - 1 - l)] : -1;
+    }
+    if (err) atomicOr(status, err);
+}
+
 }  // namespace
 }  // namespace fsta
 
@@ -377,6 +423,26 @@ extern "C" int fsta_lineage_from_parents(const int64_t* parent, int64_t n_nodes,
     if (n_nodes == 0) return FSTA_OK;
     if (!parent || !level_lookup || !status)
         return fail(FSTA_EINVAL, "fsta_lineage_from_parents: null pointer");
+    if (lineage && n_nodes <= 16384 && width <= 8192) {
+        // rows of the output staged in LDS: as many nodes per workgroup as fit, in whole waves
+        const size_t fixed = (size_t)n_nodes * 4;
+        int rows_per_wg = (int)((160 * 1024 - fixed) / ((size_t)width * 4 + 4));
+        rows_per_wg = rows_per_wg >= kThreads ? kThreads : rows_per_wg / 64 * 64;
+        // small trees: still enough workgroups to spread the walks over the CUs
+        while (rows_per_wg > 64 && (n_nodes + rows_per_wg - 1) / rows_per_wg < 16) rows_per_wg -= 64;
+        if (rows_per_wg >= 64) {
+            const size_t lds = fixed + (size_t)rows_per_wg * ((size_t)width * 4 + 4);
+            if (lds > 64 * 1024) {
+                const int rc = allow_full_lds<&lineage_rows_kernel>();
+                if (rc != FSTA_OK) return rc;
+            }
+            const unsigned wgs = (unsigned)((n_nodes + rows_per_wg - 1) / rows_per_wg);
+            hipLaunchKernelGGL(lineage_rows_kernel, dim3(wgs), dim3(kThreads), lds, static_cast<hipStream_t>(stream),
+                               parent, (int)n_nodes, (int)width, rows_per_wg, lineage, level_lookup, status);
+            FSTA_HIP_OK(hipGetLastError());
+            return FSTA_OK;
+        }
+    }
     const unsigned grid = (unsigned)((n_nodes + kThreads - 1) / kThreads);
     const int lds_nodes = n_nodes <= 16384 ? (int)n_nodes : 0;   // 64 KB of int32
     hipLaunchKernelGGL(lineage_from_parents_kernel, dim3(grid), dim3(kThreads), (size_t)lds_nodes * 4,

@@ -131,8 +131,10 @@ def test_packed_mask_matches_bool_mask():
 
 
 def test_lineage_from_parents_on_gpu():
-    for seed, window in [(1, None), (2, 8), (3, 64)]:
-        parent = trees.random_recursive_parents(777, seed, window)
+    # (up to 16384 nodes the output rows are staged in LDS; larger trees are walked row by row)
+    for seed, window, n in [(1, None, 777), (2, 8, 777), (3, 64, 777), (4, 2, 3000), (5, 40, 16384),
+                            (6, 300, 20000)]:
+        parent = trees.random_recursive_parents(n, seed, window)
         parent[::97] = -1
         want_lin, want_lvl = trees.lineage_from_parents(parent)
         lin, lvl = lineage_from_parents_gpu(torch.from_numpy(parent).cuda())
