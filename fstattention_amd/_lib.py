@@ -7,7 +7,7 @@ from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_uint3
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libfsta.so")
 
-F32, F16, BF16 = 0, 1, 2
+F32, F16, BF16, F64 = 0, 1, 2, 3
 OK, EINVAL, EUNSUPPORTED, EHIP = 0, -1, -2, -3
 FLAG_FAST_PV, FLAG_GENERIC, FLAG_WIDE_WAVES = 1, 2, 4
 
@@ -18,6 +18,7 @@ def flag_key_splits(n: int) -> int:
 
 
 PRE_TOO_MANY_ANCESTORS, PRE_BAD_NODE_ID, PRE_BAD_LEVEL = 1, 2, 4
+TREE_NOT_PREFIX_CLOSED = 8
 ABI_VERSION = 1
 
 # name -> (restype, argtypes); every symbol include/fsta.h declares
@@ -43,6 +44,7 @@ SIGNATURES = {
                                           c_void_p]),
     "fsta_dfs_order": (c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_void_p]),
+    "fsta_medusa_tree": (c_int, [c_void_p, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p]),
     "fsta_merge_states": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                                   c_int32, c_int32, c_void_p]),
 }

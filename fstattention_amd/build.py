@@ -22,6 +22,7 @@ SOURCES = [
     "fsta_capi.hip",
     "fsta_precompute.hip",
     "fsta_tree_order.hip",
+    "fsta_tree_build.hip",
     "fsta_merge.hip",
     "fsta_attention_generic.hip",
     "fsta_attention_mfma.hip",

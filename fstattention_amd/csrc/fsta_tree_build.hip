@@ -1,0 +1,248 @@
+// Draft-head probabilities -> parent array of the tree of the most probable candidate paths
+// (a Medusa-style tree), in one workgroup and launch, so that a tree that changes every decoding
+// step is built without leaving the device or the stream (the reference builds its trees on the
+// host, utils.py:27-77; README.md:16 rebuilds the kernel inputs once per step).
+//
+// A candidate is a path of ranks (r1..rd), 1 <= d <= depths, 0 <= r < topk; it scores
+// probs[0][r1] * probs[1][r2] * ... (float64, multiplied left to right).  Candidates are indexed
+// by (depth, ranks) ascending: index = start[d] + value, value = the ranks read as a base-topk
+// number.  The n-1 best candidates are kept, ties going to the smaller index; node 0 is the empty
+// path, the kept candidates are numbered 1.. in index order (so parent < child), and the parent
+// of a path is the path without its last rank.
+//
+//   1. scores of all candidates into LDS
+//   2. the (n-1)-th largest score by radix selection on the bit patterns (8 passes of 8 bits;
+//      non-negative doubles order like their bit patterns)
+//   3. "kept" flags (above the threshold, or equal to it and among the first ties), numbered by
+//      a prefix sum over the candidate index
+//   4. parent ids through the numbering of the parents' candidates
+#include "fsta_common.h"
+
+namespace fsta {
+namespace {
+
+constexpr int kBuildThreads = 1024;
+constexpr int kBuildWaves = kBuildThreads / 64;
+constexpr int kBuildRows = 16;                                  // candidate c belongs to thread c % 1024, row c / 1024
+constexpr int kBuildMaxCand = kBuildThreads * kBuildRows;       // 16384: 128 KB of scores
+constexpr int kBuildMaxProbs = 1024;                            // depths * topk
+
+template <typename T>
+__global__ __launch_bounds__(kBuildThreads) void medusa_tree_kernel(const T* __restrict__ probs, int depths, int topk,
+                                                                    int n_cand, int keep, int64_t* __restrict__ parent,
+                                                                    uint32_t* __restrict__ status) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char build_s[];
+    uint64_t* key_s = reinterpret_cast<uint64_t*>(build_s);                    // [n_cand] score bits, later node ids
+    double* prob_s = reinterpret_cast<double*>(key_s + n_cand);                // [depths * topk]
+    uint32_t* hist_s = reinterpret_cast<uint32_t*>(prob_s + depths * topk);    // [256] bytes; later counts per (row, wave)
+    uint32_t* misc_s = hist_s + 256;   // [0] chosen byte, [1] candidates still wanted
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int rows = (n_cand + kBuildThreads - 1) / kBuildThreads;
+
+    if (keep == 0) {      // the root alone
+        if (tid == 0) parent[0] = -1;
+        return;
+    }
+    for (int e = tid; e < depths * topk; e += kBuildThreads) prob_s[e] = (double)probs[e];
+    if (tid < 2) misc_s[tid] = 0u;
+    __syncthreads();
+
+    // 1. scores, depth by depth: a path's score is its prefix's score times the probability of
+    //    its last rank (the left-to-right product); one division by topk per candidate, done as
+    //    a multiplication by 2^32 / topk rounded up (exact below 2^32 / topk, i.e. for every index here)
+    if (topk == 1) {       // a single chain: one path per depth
+        if (tid == 0) {
+            double score = 1.0;
+            for (int d = 0; d < depths; ++d) {
+                score *= prob_s[d];
+                key_s[d] = (uint64_t)__double_as_longlong(score);
+            }
+        }
+        __syncthreads();
+    } else {
+        const uint32_t magic = (uint32_t)((0x100000000ull + (uint32_t)topk - 1u) / (uint32_t)topk);
+        int start = 0, prev_start = 0, count = topk;
+        for (int d = 0; start < n_cand; ++d) {
+            for (int v = tid; v < count; v += kBuildThreads) {
+                const uint32_t q = __umulhi((uint32_t)v, magic);          // v / topk
+                const uint32_t r = (uint32_t)v - q * (uint32_t)topk;
+                const double head = d == 0 ? 1.0 : __longlong_as_double((long long)key_s[prev_start + q]);
+                key_s[start + v] = (uint64_t)__double_as_longlong(head * prob_s[d * topk + r]);
+            }
+            __syncthreads();
+            prev_start = start;
+            start += count;
+            count *= topk;
+        }
+    }
+
+    // 2. threshold = the keep-th largest key
+    uint64_t prefix = 0ull;        // the bytes of the threshold found so far (in place, lower bytes zero)
+    uint32_t want = (uint32_t)keep;
+    for (int shift = 56; shift >= 0; shift -= 8) {
+        if (tid < 256) hist_s[tid] = 0u;
+        __syncthreads();
+        const uint64_t high_mask = shift == 56 ? 0ull : ~0ull << (shift + 8);
+#pragma unroll 1
+        for (int k = 0; k < rows; ++k) {
+            const int c = tid + k * kBuildThreads;
+            const uint64_t key = c < n_cand ? key_s[c] : 0ull;
+            const bool in = c < n_cand && (key & high_mask) == prefix;
+            const uint32_t bin = (uint32_t)(key >> shift) & 255u;
+            // The leading bytes of the scores are nearly all alike: 64 atomics of a wave would queue
+            // on one or two words.  For up to two byte values one lane counts for all lanes that
+            // hold it; what is left after that is spread over many words and goes lane by lane.
+            uint64_t voters = __ballot(in);
+#pragma unroll
+            for (int round = 0; round < 2; ++round) {
+                if (voters != 0ull) {
+                    const int leader = __ffsll((long long)voters) - 1;
+                    const uint32_t first = __builtin_amdgcn_readlane(bin, leader);
+                    const uint64_t same = __ballot(in && bin == first);
+                    if (lane == leader) atomicAdd(&hist_s[first], (uint32_t)__popcll(same));
+                    voters &= ~same;
+                }
+            }
+            if ((voters >> lane) & 1ull) atomicAdd(&hist_s[bin], 1u);
+        }
+        __syncthreads();
+        if (tid < 64) {
+            // lane l owns bins 255 - 4l .. 252 - 4l; counts accumulate from the largest byte down
+            uint32_t mine[4], local = 0u;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) { mine[b] = hist_s[255 - 4 * tid - b]; local += mine[b]; }
+            uint32_t incl = local;
+#pragma unroll
+            for (int dlt = 1; dlt < 64; dlt <<= 1) {
+                const uint32_t up = __shfl_up(incl, dlt, 64);
+                if (tid >= dlt) incl += up;
+            }
+            uint32_t before = incl - local;       // candidates in larger bins
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                if (before < want && want <= before + mine[b]) {
+                    misc_s[0] = (uint32_t)(255 - 4 * tid - b);
+                    misc_s[1] = want - before;
+                }
+                before += mine[b];
+            }
+        }
+        __syncthreads();
+        prefix |= (uint64_t)misc_s[0] << shift;
+        want = misc_s[1];
+    }
+    // prefix = the threshold; `want` of the candidates equal to it are kept, the first ones by index
+    const uint64_t threshold = prefix;
+
+    // 3. numbering of the kept candidates in index order.  Index order = row by row, wave by wave,
+    //    lane by lane: counts per (row, wave) from ballots (above the threshold | equal to it << 16),
+    //    an exclusive scan over those 256 counts, and the lanes below within the wave.
+    uint32_t* count_s = hist_s;
+    __syncthreads();
+#pragma unroll 1
+    for (int k = 0; k < kBuildRows; ++k) {
+        const int c = tid + k * kBuildThreads;
+        const uint64_t key = c < n_cand ? key_s[c] : 0ull;
+        const uint64_t over = __ballot(c < n_cand && key > threshold);
+        const uint64_t tie = __ballot(c < n_cand && key == threshold);
+        if (lane == 0) count_s[k * kBuildWaves + wave] = (uint32_t)__popcll(over) | ((uint32_t)__popcll(tie) << 16);
+    }
+    __syncthreads();
+    if (tid < 64) {
+        uint32_t mine[4], local = 0u;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) { mine[b] = count_s[4 * tid + b]; local += mine[b]; }
+        uint32_t incl = local;        // n_cand <= 16384: no carry between the halves
+#pragma unroll
+        for (int dlt = 1; dlt < 64; dlt <<= 1) {
+            const uint32_t up = __shfl_up(incl, dlt, 64);
+            if (tid >= dlt) incl += up;
+        }
+        uint32_t before = incl - local;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) { count_s[4 * tid + b] = before; before += mine[b]; }
+    }
+    __syncthreads();
+    const uint64_t below = (1ull << lane) - 1ull;
+#pragma unroll 1
+    for (int k = 0; k < rows; ++k) {
+        const int c = tid + k * kBuildThreads;
+        const uint64_t key = c < n_cand ? key_s[c] : 0ull;
+        const bool is_over = c < n_cand && key > threshold, is_tie = c < n_cand && key == threshold;
+        const uint64_t over = __ballot(is_over);
+        const uint64_t tie = __ballot(is_tie);
+        const uint32_t base = count_s[k * kBuildWaves + wave];
+        const uint32_t above_before = (base & 0xffffu) + (uint32_t)__popcll(over & below);
+        const uint32_t equal_before = (base >> 16) + (uint32_t)__popcll(tie & below);
+        // kept candidates before this one: those above the threshold and the kept ties
+        const bool kept = is_over || (is_tie && equal_before < want);
+        // node ids (0 = not kept) take the place of the scores
+        if (c < n_cand) key_s[c] = kept ? 1u + above_before + min(equal_before, want) : 0u;
+    }
+    __syncthreads();
+
+    // 4. parents
+    if (tid == 0) parent[0] = -1;
+    bool broken = false;
+#pragma unroll 1
+    for (int c = tid; c < n_cand; c += kBuildThreads) {
+        const uint32_t id = (uint32_t)key_s[c];
+        if (id == 0u) continue;
+        int start = 0, count = topk, prev_start = 0;
+        while (c >= start + count) { prev_start = start; start += count; count *= topk; }
+        int64_t par = 0;      // paths of one rank hang off the root
+        if (start > 0) {
+            par = (int64_t)(uint32_t)key_s[prev_start + (c - start) / topk];
+            if (par == 0) broken = true;     // the parent path was not kept: probabilities above 1 or not numbers
+        }
+        parent[id] = par;
+    }
+    if (broken) atomicOr(status, FSTA_TREE_NOT_PREFIX_CLOSED);
+}
+
+}  // namespace
+}  // namespace fsta
+
+using namespace fsta;
+
+extern "C" int fsta_medusa_tree(const void* probs, int32_t probs_dtype, int32_t depths, int32_t topk, int32_t n_nodes,
+                                int64_t* parent, uint32_t* status, void* stream) {
+    if (depths < 1 || topk < 1 || n_nodes < 1)
+        return fail(FSTA_EINVAL, "fsta_medusa_tree: depths=%d topk=%d n_nodes=%d", depths, topk, n_nodes);
+    if (probs_dtype != FSTA_F32 && probs_dtype != FSTA_F64)
+        return fail(FSTA_EINVAL, "fsta_medusa_tree: probs_dtype=%d (float32 or float64)", probs_dtype);
+    int64_t n_cand = 0, level = 1;
+    for (int d = 0; d < depths; ++d) {
+        level *= topk;
+        n_cand += level;
+        if (n_cand > kBuildMaxCand) break;
+    }
+    if (n_cand > kBuildMaxCand || (int64_t)depths * topk > kBuildMaxProbs)
+        return fail(FSTA_EUNSUPPORTED, "fsta_medusa_tree: depths=%d topk=%d give more than %d candidate paths",
+                    depths, topk, kBuildMaxCand);
+    if (n_nodes - 1 > n_cand)
+        return fail(FSTA_EINVAL, "fsta_medusa_tree: n_nodes=%d but only %lld candidate paths (+ the root)", n_nodes,
+                    (long long)n_cand);
+    if (!probs || !parent || !status) return fail(FSTA_EINVAL, "fsta_medusa_tree: null pointer");
+    const size_t lds = (size_t)n_cand * 8 + (size_t)depths * topk * 8 + (256 + 4) * 4;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (probs_dtype == FSTA_F32) {
+        if (lds > 64 * 1024) {
+            const int rc = allow_full_lds<&medusa_tree_kernel<float>>();
+            if (rc != FSTA_OK) return rc;
+        }
+        hipLaunchKernelGGL(medusa_tree_kernel<float>, dim3(1), dim3(kBuildThreads), lds, s,
+                           static_cast<const float*>(probs), depths, topk, (int)n_cand, n_nodes - 1, parent, status);
+    } else {
+        if (lds > 64 * 1024) {
+            const int rc = allow_full_lds<&medusa_tree_kernel<double>>();
+            if (rc != FSTA_OK) return rc;
+        }
+        hipLaunchKernelGGL(medusa_tree_kernel<double>, dim3(1), dim3(kBuildThreads), lds, s,
+                           static_cast<const double*>(probs), depths, topk, (int)n_cand, n_nodes - 1, parent, status);
+    }
+    FSTA_HIP_OK(hipGetLastError());
+    return FSTA_OK;
+}

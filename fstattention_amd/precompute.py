@@ -154,17 +154,19 @@ def renumber_parents_gpu(parent: torch.Tensor, perm: torch.Tensor, rank: torch.T
     return torch.where(old_parent >= 0, rank.index_select(0, old_parent.clamp(min=0)), old_parent)
 
 
-def medusa_parents_gpu(probs: torch.Tensor, n: int) -> torch.Tensor:
+def medusa_parents_gpu(probs: torch.Tensor, n: int, check: bool = False) -> torch.Tensor:
     """``probs [depths, topk]`` on the GPU -> parent array int64 ``[n]`` on the GPU, no host round trip.
 
     Device version of ``trees.medusa_parents_from_probs`` (same selection, same tie-breaks, same
     numbering): a path of ranks ``(r1..rd)`` scores the product of its ranks' probabilities, the
     ``n-1`` best paths are kept (ties: shallower first, then smaller ranks) and numbered by
     ``(depth, ranks)``; node 0 is the empty path.  Scores are formed in float64 in the host
-    version's multiplication order.  Plain torch tensor operations on the current stream; with
-    ``dfs_order_gpu``, ``lineage_from_parents_gpu(width=depths + 1)`` and
-    ``create_fst_attention_kernel_inputs(check=False)`` a tree goes from draft-head
-    probabilities to kernel inputs without touching the host.
+    version's multiplication order.  One launch of a HIP kernel on the current stream
+    (``fsta_medusa_tree``; up to 16384 candidate paths, beyond that the same steps run as torch
+    tensor operations); with ``dfs_order_gpu``, ``lineage_from_parents_gpu(width=depths + 1)`` and
+    ``create_fst_attention_kernel_inputs(check=False)`` a tree goes from draft-head probabilities
+    to kernel inputs without touching the host.  ``check`` synchronises and raises when a kept
+    path's prefix was not kept (probabilities above 1 or not numbers).
     """
     if probs.dim() != 2 or not probs.is_cuda:
         raise ValueError("probs must be a [depths, topk] tensor on the GPU")
@@ -172,6 +174,26 @@ def medusa_parents_gpu(probs: torch.Tensor, n: int) -> torch.Tensor:
     total = sum(topk ** d for d in range(1, depths + 1))
     if not 1 <= n <= total + 1:
         raise ValueError(f"n={n} outside [1, {total + 1}] for depths={depths}, topk={topk}")
+    if total > 16384 or depths * topk > 1024:
+        return _medusa_parents_torch(probs, n)
+    if probs.dtype not in (torch.float32, torch.float64):
+        probs = probs.to(torch.float64)
+    probs = probs.contiguous()
+    lib = _lib.load()
+    dev = probs.device
+    parent = torch.empty((n,), dtype=torch.int64, device=dev)
+    status = torch.zeros((1,), dtype=torch.int32, device=dev)
+    with _on_device(dev):
+        _lib.check(lib.fsta_medusa_tree(probs.data_ptr(), _lib.F32 if probs.dtype == torch.float32 else _lib.F64,
+                                        depths, topk, n, parent.data_ptr(), status.data_ptr(), _stream_ptr(dev)))
+    if check and int(status.item()) & _lib.TREE_NOT_PREFIX_CLOSED:
+        raise ValueError("the kept paths are not closed under prefixes (probabilities above 1 or not numbers)")
+    return parent
+
+
+def _medusa_parents_torch(probs: torch.Tensor, n: int) -> torch.Tensor:
+    """The steps of ``fsta_medusa_tree`` as torch tensor operations (any number of candidate paths)."""
+    depths, topk = probs.shape
     probs = probs.to(torch.float64)
     dev = probs.device
     # all paths in (depth, ranks) order: level d is the outer product of level d-1 with probs[d-1]

@@ -27,6 +27,7 @@ extern "C" {
 #define FSTA_F32  0
 #define FSTA_F16  1
 #define FSTA_BF16 2
+#define FSTA_F64  3  /* fsta_medusa_tree's probabilities only */
 
 /* return codes */
 #define FSTA_OK            0
@@ -52,6 +53,9 @@ extern "C" {
 #define FSTA_PRE_TOO_MANY_ANCESTORS 1u /* a block has more than max_ancestors unique ancestors */
 #define FSTA_PRE_BAD_NODE_ID        2u /* lineage entry < -1 or >= n_nodes                      */
 #define FSTA_PRE_BAD_LEVEL          4u /* level_lookup entry outside [-width, width)            */
+/* bit of the status word written by fsta_medusa_tree */
+#define FSTA_TREE_NOT_PREFIX_CLOSED 8u /* a kept path's parent path was not kept (probabilities
+                                          above 1 or not numbers)                                */
 
 int fsta_abi_version(void);
 
@@ -198,6 +202,26 @@ int fsta_dfs_order(const int64_t* parent, int64_t n_nodes, int32_t light_first, 
 int fsta_merge_states(const void* o_a, const float* lse_a, const void* o_b, const float* lse_b,
                       void* o_out, float* lse_out, int64_t rows, int32_t head_dim, int32_t dtype,
                       void* stream);
+
+/*
+ * Draft-head probabilities -> parent array of the tree of the most probable candidate
+ * paths (a Medusa-style static tree), on the device.  No counterpart in the reference,
+ * which builds its trees on the host (utils.py:27-77); with fsta_dfs_order,
+ * fsta_lineage_from_parents and fsta_precompute a tree goes from model output to
+ * kernel inputs on the stream, without a host round trip (README.md:16: the inputs
+ * are rebuilt once per decoding step).
+ *   probs [depths, topk] float32 or float64 (probs_dtype FSTA_F32 / FSTA_F64), row d
+ *   = probabilities of the ranked candidates of draft depth d, descending.
+ * A path of ranks (r1..rd) scores probs[0][r1] * ... * probs[d-1][rd] (float64,
+ * left to right).  Node 0 is the empty path; the other n_nodes - 1 nodes are the
+ * best-scoring paths (ties: shallower first, then smaller ranks), numbered by
+ * (depth, ranks) ascending, so parent[i] < i.  parent [n_nodes] int64, -1 for the
+ * root.  `status` (zero on entry) gets FSTA_TREE_NOT_PREFIX_CLOSED where a kept
+ * path's prefix is not kept.  At most 16384 candidate paths (sum of topk^d) and
+ * depths * topk <= 1024; n_nodes - 1 must not exceed the number of paths.
+ */
+int fsta_medusa_tree(const void* probs, int32_t probs_dtype, int32_t depths, int32_t topk,
+                     int32_t n_nodes, int64_t* parent, uint32_t* status, void* stream);
 
 #ifdef __cplusplus
 }

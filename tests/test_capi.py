@@ -35,7 +35,9 @@ def test_constants_match_header():
     text = open(HEADER).read()
     defs = dict(re.findall(r"#define\s+(FSTA_[A-Z_0-9]+)\s+(-?\d+)u?\b", text))
     assert int(defs["FSTA_ABI_VERSION"]) == _lib.ABI_VERSION
-    assert (int(defs["FSTA_F32"]), int(defs["FSTA_F16"]), int(defs["FSTA_BF16"])) == (_lib.F32, _lib.F16, _lib.BF16)
+    assert (int(defs["FSTA_F32"]), int(defs["FSTA_F16"]), int(defs["FSTA_BF16"]), int(defs["FSTA_F64"])) == \
+        (_lib.F32, _lib.F16, _lib.BF16, _lib.F64)
+    assert int(defs["FSTA_TREE_NOT_PREFIX_CLOSED"]) == _lib.TREE_NOT_PREFIX_CLOSED
     assert (int(defs["FSTA_OK"]), int(defs["FSTA_EINVAL"]), int(defs["FSTA_EUNSUPPORTED"]),
             int(defs["FSTA_EHIP"])) == (_lib.OK, _lib.EINVAL, _lib.EUNSUPPORTED, _lib.EHIP)
     assert (int(defs["FSTA_FLAG_FAST_PV"]), int(defs["FSTA_FLAG_GENERIC"]), int(defs["FSTA_FLAG_WIDE_WAVES"])) == \
@@ -77,6 +79,17 @@ def test_argument_validation_happens_before_any_gpu_work():
     assert lib.fsta_merge_states(None, None, None, None, None, None, 0, 64, _lib.BF16, None) == _lib.OK       # nothing to do
     with pytest.raises(_lib.FstaError):
         _lib.check(_lib.EINVAL)
+
+
+def test_tree_builder_rejects_bad_arguments_before_any_gpu_work():
+    lib = _lib.load()
+    call = lambda *a: lib.fsta_medusa_tree(*a)
+    assert call(8, _lib.F64, 0, 10, 5, 8, 8, None) == _lib.EINVAL
+    assert call(8, _lib.BF16, 4, 10, 5, 8, 8, None) == _lib.EINVAL and b"probs_dtype" in lib.fsta_last_error()
+    assert call(8, _lib.F64, 4, 12, 5, 8, 8, None) == _lib.EUNSUPPORTED      # 22620 candidate paths
+    assert call(8, _lib.F64, 2, 600, 5, 8, 8, None) == _lib.EUNSUPPORTED     # 1200 probabilities
+    assert call(8, _lib.F64, 2, 3, 14, 8, 8, None) == _lib.EINVAL            # 12 paths + root < 14 nodes
+    assert call(None, _lib.F64, 2, 3, 5, 8, 8, None) == _lib.EINVAL and b"null" in lib.fsta_last_error()
 
 
 def test_workspace_planning_is_host_arithmetic():

@@ -194,6 +194,29 @@ def test_medusa_tree_built_on_the_gpu_matches_the_host_builder():
         np.testing.assert_array_equal(got.cpu().numpy(), want)
     with pytest.raises(ValueError):
         medusa_parents_gpu(torch.ones((2, 3)).cuda(), 14)     # only 3 + 9 paths + root exist
+    # ties everywhere (the candidate order decides), every path kept, one rank per depth, float32 input
+    uniform = np.full((3, 6), 0.125)
+    for n in (2, 7, 8, 30, 100, 6 + 36 + 216 + 1):
+        np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(uniform).cuda(), n).cpu().numpy(),
+                                      trees.medusa_parents_from_probs(uniform, n))
+    halves = np.array([[0.5, 0.25, 0.25], [0.5, 0.5, 0.0], [1.0, 0.0, 0.0]])     # products tie across depths
+    for n in range(1, 3 + 9 + 27 + 2):
+        np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(halves).cuda(), n).cpu().numpy(),
+                                      trees.medusa_parents_from_probs(halves, n))
+    chain = np.array([[0.9], [0.8], [0.7], [0.6], [0.5]])
+    np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(chain).cuda(), 6).cpu().numpy(),
+                                  np.array([-1, 0, 1, 2, 3, 4]))
+    p32 = trees.medusa_probs(4, 10, 0.3, 11).astype(np.float32)
+    np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(p32).cuda(), 200).cpu().numpy(),
+                                  trees.medusa_parents_from_probs(p32, 200))
+    big = trees.medusa_probs(4, 11, 0.3, 12)       # 16104 candidate paths: the largest the kernel takes
+    np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(big).cuda(), 1000).cpu().numpy(),
+                                  trees.medusa_parents_from_probs(big, 1000))
+    wide = trees.medusa_probs(2, 200, 0.3, 13)     # 40200 paths: tensor operations instead of the kernel
+    np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(wide).cuda(), 300).cpu().numpy(),
+                                  trees.medusa_parents_from_probs(wide, 300))
+    with pytest.raises(ValueError):                # a deeper path scoring above its prefix
+        medusa_parents_gpu(torch.tensor([[0.5, 0.1], [3.0, 0.1]], dtype=torch.float64).cuda(), 2, check=True)
 
 
 def test_device_only_pipeline_from_probabilities_to_kernel_inputs():
