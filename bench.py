@@ -253,6 +253,53 @@ def time_precompute(wl, reps=50):
     return (time.perf_counter() - t0) / reps
 
 
+def time_front_end(index, reps=20):
+    """Device microseconds of the per-step tree front-end of configuration `index`, each stage
+    recorded `reps` times into a HIP graph (allocations of the Python wrappers included, host time not):
+    draft probabilities -> parent array (cfg2's generator only), depth-first order, parent array ->
+    lineage, lineage -> kernel inputs."""
+    import torch
+    from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, lineage_from_parents_gpu,
+                                  medusa_parents_gpu, trees)
+    dev = torch.device("cuda", 0)
+    cfg = trees.config(index)
+    parent = torch.from_numpy(cfg.parent).to(dev)
+    lineage, level = trees.lineage_from_parents(cfg.parent)
+    lineage, level = lineage.to(dev), level.to(dev)
+    width = lineage.shape[1]
+    max_anc = trees.required_max_ancestors(cfg.parent, cfg.block_m, 16)
+
+    def device_us(fn):
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            for _ in range(3):
+                fn()
+            stream.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for _ in range(reps):
+                    fn()
+            graph.replay()
+            stream.synchronize()
+            ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            ev0.record(stream)
+            graph.replay()
+            ev1.record(stream)
+            torch.cuda.synchronize()
+        return round(ev0.elapsed_time(ev1) * 1e3 / reps, 2)
+
+    out = {
+        "dfs_order_us": device_us(lambda: dfs_order_gpu(parent, "light_first", check=False)),
+        "lineage_from_parents_us": device_us(lambda: lineage_from_parents_gpu(parent, width=width, check=False)),
+        "kernel_inputs_us": device_us(lambda: create_fst_attention_kernel_inputs(
+            lineage, level, cfg.block_m, max_anc, mutate_lineage=False, check=False, want_bool_mask=False)),
+    }
+    if index == 2:
+        probs = torch.from_numpy(trees.medusa_probs()).to(dev)
+        out["tree_from_probabilities_us"] = device_us(lambda: medusa_parents_gpu(probs, cfg.n_nodes))
+    return out
+
+
 def cpu_baseline(wl, budget_s=10.0):
     """The oracle's dense-masked attention (reference fstattention.py:214-219 restated for
     the CPU, float32 arithmetic on the bf16-rounded inputs) on the host cores."""
@@ -456,6 +503,10 @@ def main():
             }
             del w
             torch.cuda.empty_cache()
+        # the integer kernels that turn a new tree into kernel inputs once per decoding step
+        extra["front_end_device_us"] = {trees_name: time_front_end(idx) for idx, trees_name in
+                                        ((2, "cfg2_medusa256"), (3, "cfg3_deep1024"), (4, "cfg4_wide4096"),
+                                         (5, "cfg5_batched2048"))}
         # the headline tree behind a shared prefix (the KV cache of a decoding step, reference
         # fstattention.py:113-136): the prefix as each block's own loop, and cut into runs of keys
         for prefix in (4096, 16384):

@@ -439,6 +439,49 @@ def test_hip_graph_replays_match_eager_calls():
     assert_close(out, want, cfg.dtype, "last replay")
 
 
+def test_decoding_step_from_probabilities_in_one_graph():
+    """Draft-head probabilities -> tree -> depth-first order -> lineage -> kernel inputs -> attention,
+    captured once as one HIP graph; every replay reads new probabilities (a different tree) and new
+    q/k/v from the same buffers and must match the host-built tree and the oracle."""
+    from fstattention_amd import medusa_parents_gpu
+    n, depths, topk, m, d, max_anc = 256, 4, 10, 64, 128, 64
+    scale = 1.0 / math.sqrt(d)
+    probs = torch.from_numpy(trees.medusa_probs(depths, topk, 0.3, 50)).cuda()
+    q, k, v = (t.cuda() for t in rand_qkv(1, 2, n, n, d, torch.bfloat16, 50))
+
+    def step():
+        parent = medusa_parents_gpu(probs, n)
+        perm, rank = dfs_order_gpu(parent, "light_first", check=False)
+        new_parent = renumber_parents_gpu(parent, perm, rank)
+        lineage, level = lineage_from_parents_gpu(new_parent, width=depths + 1, check=False)
+        *inputs, status = create_fst_attention_kernel_inputs(lineage, level, m, max_anc, check=False,
+                                                             want_bool_mask=False)
+        # tokens arrive in the builder's numbering: into depth-first order and back around the op
+        o = fst_attention(q.index_select(2, perm), k.index_select(2, perm), v.index_select(2, perm), *inputs,
+                          scale, BLOCK_M=m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32)
+        return o.index_select(2, rank), parent, status
+
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        step()
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            out, parent, status = step()
+    for replay in range(3):
+        probs.copy_(torch.from_numpy(trees.medusa_probs(depths, topk, 0.3, 60 + replay)))
+        g = torch.Generator().manual_seed(70 + replay)
+        q.copy_(torch.randn(q.shape, generator=g).to(q.dtype))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want_parent = trees.medusa_parents_from_probs(probs.cpu().numpy(), n)
+        np.testing.assert_array_equal(parent.cpu().numpy(), want_parent)
+        assert int(status.item()) == 0
+        want, _ = dense_oracle(q.cpu(), k.cpu(), v.cpu(), want_parent, scale)
+        assert_close(out, want, torch.bfloat16, f"replay {replay}")
+
+
 def test_two_host_threads_on_their_own_streams():
     """Entry points keep no state between calls: two threads, each with its own stream, inputs and
     tree, launching at the same time get their own results."""
