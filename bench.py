@@ -75,6 +75,7 @@ class Workload:
 
         self.torch = torch
         self.cfg = cfg = trees.config(index, dtype)
+        self.cfg_index = index
         if order is not None:
             # the same tree with its nodes (tokens) numbered depth-first (reference README.md:19-20)
             import dataclasses
@@ -330,6 +331,14 @@ def cpu_baseline(wl, budget_s=10.0):
     med = times[len(times) // 2]
     scale_up = (wl.z * wl.h) / heads      # slices not run: time extrapolated linearly
     per_call = med * scale_up
+    # the per-tree precompute (reference utils.py:104-129) restated in numpy, beside the HIP kernel
+    lin, lvl = wl.lineage.cpu().numpy(), wl.level.cpu().numpy()
+    pre = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        tree_precompute.block_inputs(lin.copy(), lvl, wl.m, wl.max_anc)
+        pre.append(time.perf_counter() - t0)
+    pre.sort()
     return {
         "value": round(wl.kv_bytes / per_call / 1e9, 4),
         "unit": "GB/s",
@@ -339,6 +348,8 @@ def cpu_baseline(wl, budget_s=10.0):
         "sample": (f"dense-masked attention oracle, float32 on {wl.dtype}-rounded inputs, "
                    f"{heads} of {wl.z * wl.h} (batch, head) slices of the same workload, "
                    f"median of {len(times)} runs" + (", scaled linearly to all slices" if scale_up != 1 else "")),
+        "precompute_us_per_tree": {"cpu_numpy_port": round(pre[len(pre) // 2] * 1e6, 1),
+                                   "gpu_device": time_front_end(wl.cfg_index)["kernel_inputs_us"]},
     }, parity
 
 
