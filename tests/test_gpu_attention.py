@@ -400,6 +400,22 @@ def test_random_shapes_against_oracle(seed):
     run_tree(parent, block_m, z, h, d, dtype, seed, prefix=prefix, wide_waves=(seed % 8 == 5))
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes_with_key_runs_against_oracle(seed):
+    """The same draw with a shared prefix of up to 3000 keys, cut into a forced or library-chosen
+    number of runs (ragged last runs, more runs than make sense, heads that are no multiple of 8)."""
+    rng = np.random.default_rng(3000 + seed)
+    block_m = int(rng.choice([32, 64, 128]))
+    d = int(rng.choice([32, 64, 128]))
+    dtype = [torch.bfloat16, torch.float16][seed % 2]
+    n = int(rng.integers(1, 4 * block_m))
+    parent = trees.random_recursive_parents(n, seed, window=[None, 4][seed % 2])
+    prefix = int(rng.integers(33, 3000))
+    splits = [None, 2, 3, 5, 8, 13][seed % 6]
+    run_tree(parent, block_m, int(rng.integers(1, 3)), int(rng.integers(1, 6)), d, dtype, seed, prefix=prefix,
+             key_splits=splits)
+
+
 def test_hip_graph_replays_match_eager_calls():
     """The op captured into a HIP graph (precompute + attention, as a decoding step would), replayed
     several times with eager launches and synchronisations in between; every replay must give the
