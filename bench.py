@@ -39,9 +39,9 @@ INFINITY_CACHE_BYTES = 256 << 20
 
 # HBM bytes per launch of the headline kernel (256-node tree, cold buffers) from two
 # rocprofv3 --pmc runs, see profiles/attn_mfma16_kernel_cfg2_medusa256_hbm_traffic.txt:
-# FETCH_SIZE 3174.5 KiB x 2.0 (a plain 256 MiB copy reads 131084 KiB on this counter, i.e. the
+# FETCH_SIZE 3184.0 KiB x 2.0 (a plain 256 MiB copy reads 131084 KiB on this counter, i.e. the
 # counter sees half of the read traffic) + WRITE_SIZE 2080 KiB x 1.0 (the copy reads 262144).
-MEASURED_TRAFFIC_BYTES = int((3174.5 * 2 + 2080) * 1024)
+MEASURED_TRAFFIC_BYTES = int((3184.0 * 2 + 2080) * 1024)
 
 
 def parse_args():
@@ -254,7 +254,7 @@ def time_precompute(wl, reps=50):
     return (time.perf_counter() - t0) / reps
 
 
-def time_front_end(index, reps=20):
+def time_front_end(index, reps=20, stages=None):
     """Device microseconds of the per-step tree front-end of configuration `index`, each stage
     recorded `reps` times into a HIP graph (allocations of the Python wrappers included, host time not):
     draft probabilities -> parent array (cfg2's generator only), depth-first order, parent array ->
@@ -289,16 +289,16 @@ def time_front_end(index, reps=20):
             torch.cuda.synchronize()
         return round(ev0.elapsed_time(ev1) * 1e3 / reps, 2)
 
-    out = {
-        "dfs_order_us": device_us(lambda: dfs_order_gpu(parent, "light_first", check=False)),
-        "lineage_from_parents_us": device_us(lambda: lineage_from_parents_gpu(parent, width=width, check=False)),
-        "kernel_inputs_us": device_us(lambda: create_fst_attention_kernel_inputs(
-            lineage, level, cfg.block_m, max_anc, mutate_lineage=False, check=False, want_bool_mask=False)),
+    calls = {
+        "dfs_order_us": lambda: dfs_order_gpu(parent, "light_first", check=False),
+        "lineage_from_parents_us": lambda: lineage_from_parents_gpu(parent, width=width, check=False),
+        "kernel_inputs_us": lambda: create_fst_attention_kernel_inputs(
+            lineage, level, cfg.block_m, max_anc, mutate_lineage=False, check=False, want_bool_mask=False),
     }
     if index == 2:
         probs = torch.from_numpy(trees.medusa_probs()).to(dev)
-        out["tree_from_probabilities_us"] = device_us(lambda: medusa_parents_gpu(probs, cfg.n_nodes))
-    return out
+        calls["tree_from_probabilities_us"] = lambda: medusa_parents_gpu(probs, cfg.n_nodes)
+    return {name: device_us(fn) for name, fn in calls.items() if stages is None or name in stages}
 
 
 def cpu_baseline(wl, budget_s=10.0):
@@ -349,7 +349,7 @@ def cpu_baseline(wl, budget_s=10.0):
                    f"{heads} of {wl.z * wl.h} (batch, head) slices of the same workload, "
                    f"median of {len(times)} runs" + (", scaled linearly to all slices" if scale_up != 1 else "")),
         "precompute_us_per_tree": {"cpu_numpy_port": round(pre[len(pre) // 2] * 1e6, 1),
-                                   "gpu_device": time_front_end(wl.cfg_index)["kernel_inputs_us"]},
+                                   "gpu_device": time_front_end(wl.cfg_index, stages=("kernel_inputs_us",))["kernel_inputs_us"]},
     }, parity
 
 
