@@ -437,8 +437,9 @@ def main():
         "cross_check": {"max_abs_diff_vs_scalar_kernel": max_err, "tol": tol, "ok": ok},
         "roofline": {
             "bound": "hbm",
-            "kernel": ("attn_mfma16_kernel<bf16, D=128, 32-row halves of the 64-row blocks, split P, 2 key shares>" if args.config == 2 else
-                       "attn_generic_kernel" if wl.dtype == torch.float32 else "attn_mfma16_kernel"),
+            "kernel": ("attn_generic_kernel" if wl.dtype == torch.float32 else
+                       "attn_mfma16_kernel<bf16, D=128, 32-row halves of the 64-row blocks, split P, 2 key shares>"
+                       if args.config == 2 and wl.dtype == torch.bfloat16 else "attn_mfma16_kernel"),
             "achieved": round(achieved, 2),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
