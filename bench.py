@@ -331,6 +331,17 @@ def cpu_baseline(wl, budget_s=10.0):
     med = times[len(times) // 2]
     scale_up = (wl.z * wl.h) / heads      # slices not run: time extrapolated linearly
     per_call = med * scale_up
+    # the same routine in the storage type's own arithmetic (what the reference's oracle does on its
+    # fp16 tensors, fstattention.py:214-219): reported beside the float32 run, not used as the checker
+    narrow_us = None
+    if wl.dtype != torch.float32:
+        narrow = []
+        while len(narrow) < 3 or (sum(narrow) < 2.0 and len(narrow) < 50):
+            t0 = time.perf_counter()
+            dense_attention.dense_tree_attention(qs, ks, vs, mask, wl.scale, dtype=wl.dtype)
+            narrow.append(time.perf_counter() - t0)
+        narrow.sort()
+        narrow_us = round(narrow[len(narrow) // 2] * scale_up * 1e6, 1)
     # the per-tree precompute (reference utils.py:104-129) restated in numpy, beside the HIP kernel
     lin, lvl = wl.lineage.cpu().numpy(), wl.level.cpu().numpy()
     pre = []
@@ -345,6 +356,7 @@ def cpu_baseline(wl, budget_s=10.0):
         "cores": cores,
         "kind": "port",
         "us_per_call": round(per_call * 1e6, 1),
+        "us_per_call_in_storage_type_arithmetic": narrow_us,
         "sample": (f"dense-masked attention oracle, float32 on {wl.dtype}-rounded inputs, "
                    f"{heads} of {wl.z * wl.h} (batch, head) slices of the same workload, "
                    f"median of {len(times)} runs" + (", scaled linearly to all slices" if scale_up != 1 else "")),
