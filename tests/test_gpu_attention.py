@@ -73,6 +73,74 @@ def test_config5_bf16_head_subset_against_oracle(wide_waves):
              wide_waves=wide_waves)
 
 
+def sampled_rows_check(q, k, v, parent, o, lse, scale, prefix, samples, seed, dtype, what):
+    """Rows of a launch too large for the dense oracle: row i attends to the prefix, its ancestors
+    and itself, so its output is a softmax over that handful of keys (float64 on the host)."""
+    rng = np.random.default_rng(seed)
+    z_, h_, nq, d = q.shape
+    tol = TOL[dtype]
+    for _ in range(samples):
+        z, h, i = int(rng.integers(z_)), int(rng.integers(h_)), int(rng.integers(len(parent)))
+        keys, a = list(range(prefix)) + [prefix + i], int(parent[i])
+        while a >= 0:
+            keys.append(prefix + a)
+            a = int(parent[a])
+        idx = torch.tensor(keys, device=q.device)
+        s = (k[z, h].index_select(0, idx).double() @ q[z, h, i].double()) * scale
+        w = torch.softmax(s, 0)
+        want = (w[:, None] * v[z, h].index_select(0, idx).double()).sum(0)
+        got = o[z, h, i].double()
+        err = (got - want).abs()
+        assert bool((err <= tol + tol * want.abs()).all()), f"{what}: slice ({z},{h}) row {i}: max err {float(err.max()):.3e}"
+        want_lse = torch.logsumexp(s, 0) / math.log(2.0)
+        assert abs(float(lse[z * h_ + h, i]) - float(want_lse)) <= 2e-3 * max(1.0, abs(float(want_lse)))
+
+
+@pytest.mark.parametrize("order", [None, "light_first"])
+def test_config5_full_size_sampled_rows(order):
+    """All 8 x 64 slices of configuration 5 (8192 workgroups), in the given and in depth-first token
+    order; checked on sampled rows, and the two kernels against each other on one whole slice."""
+    cfg = trees.config(5)
+    parent = cfg.parent
+    if order:
+        parent, _ = trees.renumber_parents(parent, trees.dfs_order(parent, order))
+    m, d, n = cfg.block_m, cfg.head_dim, cfg.n_nodes
+    lineage, level = trees.lineage_from_parents(parent)
+    max_anc = trees.required_max_ancestors(parent, m, 16)
+    inputs = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), m, max_anc)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    q, k, v = (torch.randn((cfg.batch, cfg.heads, n, d), generator=g, device="cuda", dtype=torch.float32)
+               .to(torch.bfloat16) for _ in range(3))
+    scale = 1.0 / math.sqrt(d)
+    o, lse = fst_attention(q, k, v, *inputs, scale, BLOCK_M=m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32,
+                           return_lse=True)
+    assert bool(torch.isfinite(o).all())
+    sampled_rows_check(q, k, v, parent, o, lse, scale, 0, 96, 55, torch.bfloat16, f"cfg5 order={order}")
+    one = fst_attention(q[7:, 63:].contiguous(), k[7:, 63:].contiguous(), v[7:, 63:].contiguous(), *inputs, scale,
+                        BLOCK_M=m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32, generic=True)
+    torch.testing.assert_close(o[7:, 63:], one, atol=2e-3, rtol=2e-3)
+
+
+def test_large_tree_behind_a_long_prefix_sampled_rows():
+    """40000 tokens behind 5000 prefix keys, 3 heads: index arithmetic far beyond the benchmark sizes
+    (key runs chosen by the library), checked on sampled rows."""
+    n, prefix, m, d, h = 40000, 5000, 128, 64, 3
+    parent = trees.random_recursive_parents(n, 77, window=300)
+    lineage, level = trees.lineage_from_parents(parent)
+    max_anc = trees.required_max_ancestors(parent, m, 16)
+    a_idx, a_mask, l_idx = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), m, max_anc)
+    a_idx, l_idx = shift_for_prefix(a_idx, l_idx, prefix)
+    nq = a_idx.shape[0] * m
+    g = torch.Generator(device="cuda").manual_seed(6)
+    q = torch.randn((1, h, nq, d), generator=g, device="cuda").to(torch.float16)
+    k, v = (torch.randn((1, h, prefix + nq, d), generator=g, device="cuda").to(torch.float16) for _ in range(2))
+    scale = 1.0 / math.sqrt(d)
+    for splits in (1, None):
+        o, lse = fst_attention(q, k, v, a_idx, a_mask, l_idx, scale, BLOCK_M=m, MAX_ANCESTORS=max_anc,
+                               out_dtype=torch.float32, return_lse=True, key_splits=splits)
+        sampled_rows_check(q, k, v, parent, o, lse, scale, prefix, 48, 66, torch.float16, f"large tree splits={splits}")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("d", [16, 32, 64, 128])
 @pytest.mark.parametrize("block_m", [16, 32, 64, 128])
