@@ -16,22 +16,43 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kTileN = 32;
+constexpr int kPad = 4;     // floats of padding per LDS row: rows stay 16-byte aligned for vector reads
+
+// 16 bytes of T -> floats
+template <typename T> struct Vec16 { static constexpr int n = 16 / (int)sizeof(T); };
+template <typename T>
+__device__ __forceinline__ void load16(const T* src, float (&out)[Vec16<T>::n]) {
+    struct alignas(16) Pack { T v[Vec16<T>::n]; };
+    const Pack p = *reinterpret_cast<const Pack*>(src);
+#pragma unroll
+    for (int i = 0; i < Vec16<T>::n; ++i) out[i] = to_float(p.v[i]);
+}
 
 template <int D, int M>
 constexpr size_t generic_lds_bytes() {
-    return sizeof(float) * (size_t)(M * (D + 1) + kTileN * (D + 1) + kTileN * D + M * (kTileN + 1) + 2 * M)
+    return sizeof(float) * (size_t)(M * (D + kPad) + 2 * kTileN * (D + kPad) + M * (kTileN + kPad) + 2 * M)
            + sizeof(int) * kTileN;
 }
 
+// Register tiles: a thread owns kRowsS x 4 scores of a tile (4 neighbouring keys) and kRowsO x 4
+// output values (4 neighbouring head dims), and reads its operands from LDS 16 bytes at a time.
 template <typename T, int D, int M>
 __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
-    extern __shared__ float smem[];
-    float* q_s = smem;                        // [M][D+1]
-    float* k_s = q_s + M * (D + 1);           // [kTileN][D+1]
-    float* v_s = k_s + kTileN * (D + 1);      // [kTileN][D]
-    float* s_s = v_s + kTileN * D;            // [M][kTileN+1] scores, then weights
-    float* alpha_s = s_s + M * (kTileN + 1);  // [M] rescale of the running sums
-    float* stat_s = alpha_s + M;              // [M] 1/l for the epilogue
+    constexpr int kPitch = D + kPad;            // floats per row of q_s / k_s / v_s
+    constexpr int kPitchS = kTileN + kPad;      // floats per row of s_s
+    constexpr int kColGroupsS = kTileN / 4;     // 8 groups of 4 keys
+    constexpr int kRowSlotsS = kThreads / kColGroupsS;                 // 32 row slots
+    constexpr int kRowsS = (M + kRowSlotsS - 1) / kRowSlotsS;          // score rows per thread
+    constexpr int kColGroupsO = D / 4;          // groups of 4 head dims
+    constexpr int kRowSlotsO = kThreads / kColGroupsO;
+    constexpr int kRowsO = (M + kRowSlotsO - 1) / kRowSlotsO;          // output rows per thread
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    float* q_s = smem;                          // [M][kPitch]
+    float* k_s = q_s + M * kPitch;              // [kTileN][kPitch]
+    float* v_s = k_s + kTileN * kPitch;         // [kTileN][kPitch]
+    float* s_s = v_s + kTileN * kPitch;         // [M][kPitchS] scores, then weights
+    float* alpha_s = s_s + M * kPitchS;         // [M] rescale of the running sums
+    float* stat_s = alpha_s + M;                // [M] 1/l for the epilogue
     int* key_s = reinterpret_cast<int*>(stat_s + M);  // [kTileN] K/V row of each tile column
 
     const int tid = threadIdx.x;
@@ -42,16 +63,28 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
     const T* kb = static_cast<const T*>(p.k) + (size_t)hz * p.nk * D;
     const T* vb = static_cast<const T*>(p.v) + (size_t)hz * p.nk * D;
 
-    for (int e = tid; e < M * D; e += kThreads) {
-        const int m = e / D, d = e % D;
+    constexpr int kVec = Vec16<T>::n;           // elements per 16-byte global load
+    for (int e = tid; e < M * D / kVec; e += kThreads) {
+        const int m = e / (D / kVec), d = (e % (D / kVec)) * kVec;
         const int row = row0 + m;
-        q_s[m * (D + 1) + d] = row < p.nq ? to_float(qb[(size_t)row * D + d]) : 0.f;
+        float x[kVec];
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) x[i] = 0.f;
+        if (row < p.nq) load16(qb + (size_t)row * D + d, x);
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) q_s[m * kPitch + d + i] = x[i];
     }
 
-    constexpr int kAcc = M * D / kThreads;
-    float acc[kAcc];
+    // this thread's tiles
+    const int sc = (tid % kColGroupsS) * 4;     // first key column of the score tile
+    const int sr = tid / kColGroupsS;           // score rows sr + kRowSlotsS * i
+    const int oc = (tid % kColGroupsO) * 4;     // first head dim of the output tile
+    const int orow = tid / kColGroupsO;         // output rows orow + kRowSlotsO * i
+    float acc[kRowsO][4];
 #pragma unroll
-    for (int i = 0; i < kAcc; ++i) acc[i] = 0.f;
+    for (int i = 0; i < kRowsO; ++i)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[i][c] = 0.f;
     float m_i = -INFINITY, l_i = 0.f;  // running max / sum of row `tid` (tid < M)
 
     int n_anc = p.anc_count ? p.anc_count[j] : p.max_anc;
@@ -78,48 +111,72 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
         }
         __syncthreads();
 
-        for (int e = tid; e < kTileN * D; e += kThreads) {
-            const int n = e / D, d = e % D;
+        for (int e = tid; e < kTileN * D / kVec; e += kThreads) {
+            const int n = e / (D / kVec), d = (e % (D / kVec)) * kVec;
             const int key = key_s[n];
-            float kf = 0.f, vf = 0.f;
+            float kf[kVec], vf[kVec];
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) { kf[i] = 0.f; vf[i] = 0.f; }
             if (key >= 0) {
-                kf = to_float(kb[(size_t)key * D + d]);
-                vf = to_float(vb[(size_t)key * D + d]);
+                load16(kb + (size_t)key * D + d, kf);
+                load16(vb + (size_t)key * D + d, vf);
             }
-            k_s[n * (D + 1) + d] = kf;
-            v_s[n * D + d] = vf;
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) {
+                k_s[n * kPitch + d + i] = kf[i];
+                v_s[n * kPitch + d + i] = vf[i];
+            }
         }
         __syncthreads();
 
-        for (int e = tid; e < M * kTileN; e += kThreads) {
-            const int m = e / kTileN, n = e % kTileN;
-            bool ok = key_s[n] >= 0;
-            if (kind == 0) {
-                const uint32_t w = p.mask_bits[((size_t)j * p.mask_words + (base >> 5)) * M + m];
-                ok = ok && ((w >> n) & 1u);
-            } else if (kind == 1) {
-                ok = ok && (m == base + n);
+        // scores of this thread's tile: rows sr + 32 i, keys sc .. sc + 3
+        if (sr < M) {
+            float dot[kRowsS][4];
+#pragma unroll
+            for (int i = 0; i < kRowsS; ++i)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) dot[i][c] = 0.f;
+#pragma unroll 4
+            for (int d = 0; d < D; d += 4) {
+                float4 kq[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) kq[c] = *reinterpret_cast<const float4*>(k_s + (sc + c) * kPitch + d);
+#pragma unroll
+                for (int i = 0; i < kRowsS; ++i) {
+                    const int m = sr + kRowSlotsS * i;
+                    if (kRowsS * kRowSlotsS > M && m >= M) continue;
+                    const float4 qq = *reinterpret_cast<const float4*>(q_s + m * kPitch + d);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+                        dot[i][c] += qq.x * kq[c].x + qq.y * kq[c].y + qq.z * kq[c].z + qq.w * kq[c].w;
+                }
             }
-            float s = -INFINITY;
-            if (ok) {
-                float dot = 0.f;
-#pragma unroll 8
-                for (int d = 0; d < D; ++d) dot += q_s[m * (D + 1) + d] * k_s[n * (D + 1) + d];
-                s = dot * p.scale_log2e;
+#pragma unroll
+            for (int i = 0; i < kRowsS; ++i) {
+                const int m = sr + kRowSlotsS * i;
+                if (kRowsS * kRowSlotsS > M && m >= M) continue;
+                uint32_t w = 0xffffffffu;
+                if (kind == 0) w = p.mask_bits[((size_t)j * p.mask_words + (base >> 5)) * M + m];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int n = sc + c;
+                    bool ok = key_s[n] >= 0 && ((w >> n) & 1u);
+                    if (kind == 1) ok = ok && (m == base + n);
+                    s_s[m * kPitchS + n] = ok ? dot[i][c] * p.scale_log2e : -INFINITY;
+                }
             }
-            s_s[m * (kTileN + 1) + n] = s;
         }
         __syncthreads();
 
         if (tid < M) {
             float mx = m_i;
-            for (int n = 0; n < kTileN; ++n) mx = fmaxf(mx, s_s[tid * (kTileN + 1) + n]);
+            for (int n = 0; n < kTileN; ++n) mx = fmaxf(mx, s_s[tid * kPitchS + n]);
             const float alpha = (mx == -INFINITY) ? 1.f : exp2f(m_i - mx);
             float sum = 0.f;
             for (int n = 0; n < kTileN; ++n) {
-                const float s = s_s[tid * (kTileN + 1) + n];
+                const float s = s_s[tid * kPitchS + n];
                 const float w = (s == -INFINITY) ? 0.f : exp2f(s - mx);
-                s_s[tid * (kTileN + 1) + n] = w;
+                s_s[tid * kPitchS + n] = w;
                 sum += w;
             }
             l_i = l_i * alpha + sum;
@@ -128,14 +185,32 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
         }
         __syncthreads();
 
+        // O tile: rows orow + kRowSlotsO i, head dims oc .. oc + 3
+        if (orow < M) {
 #pragma unroll
-        for (int i = 0; i < kAcc; ++i) {
-            const int e = tid + i * kThreads;
-            const int m = e / D, d = e % D;
-            float a = acc[i] * alpha_s[m];
-#pragma unroll 8
-            for (int n = 0; n < kTileN; ++n) a += s_s[m * (kTileN + 1) + n] * v_s[n * D + d];
-            acc[i] = a;
+            for (int i = 0; i < kRowsO; ++i) {
+                const int m = orow + kRowSlotsO * i;
+                if (kRowsO * kRowSlotsO > M && m >= M) continue;
+                const float a = alpha_s[m];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) acc[i][c] *= a;
+            }
+#pragma unroll 2
+            for (int n = 0; n < kTileN; n += 4) {
+                float4 vv[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) vv[u] = *reinterpret_cast<const float4*>(v_s + (n + u) * kPitch + oc);
+#pragma unroll
+                for (int i = 0; i < kRowsO; ++i) {
+                    const int m = orow + kRowSlotsO * i;
+                    if (kRowsO * kRowSlotsO > M && m >= M) continue;
+                    const float4 w = *reinterpret_cast<const float4*>(s_s + m * kPitchS + n);
+                    acc[i][0] += w.x * vv[0].x + w.y * vv[1].x + w.z * vv[2].x + w.w * vv[3].x;
+                    acc[i][1] += w.x * vv[0].y + w.y * vv[1].y + w.z * vv[2].y + w.w * vv[3].y;
+                    acc[i][2] += w.x * vv[0].z + w.y * vv[1].z + w.z * vv[2].z + w.w * vv[3].z;
+                    acc[i][3] += w.x * vv[0].w + w.y * vv[1].w + w.z * vv[2].w + w.w * vv[3].w;
+                }
+            }
         }
         __syncthreads();
     }
@@ -148,17 +223,21 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
     }
     __syncthreads();
 
+    if (orow < M) {
 #pragma unroll
-    for (int i = 0; i < kAcc; ++i) {
-        const int e = tid + i * kThreads;
-        const int m = e / D, d = e % D;
-        const int row = row0 + m;
-        if (row >= p.nq) continue;
-        const float l = stat_s[m];
-        const float val = l > 0.f ? acc[i] / l : 0.f;
-        const size_t off = ((size_t)hz * p.nq + row) * D + d;
-        if (p.out_f32) static_cast<float*>(p.o)[off] = val;
-        else static_cast<T*>(p.o)[off] = from_float<T>(val);
+        for (int i = 0; i < kRowsO; ++i) {
+            const int m = orow + kRowSlotsO * i;
+            const int row = row0 + m;
+            if ((kRowsO * kRowSlotsO > M && m >= M) || row >= p.nq) continue;
+            const float l = stat_s[m];
+            const size_t off = ((size_t)hz * p.nq + row) * D + oc;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const float val = l > 0.f ? acc[i][c] / l : 0.f;
+                if (p.out_f32) static_cast<float*>(p.o)[off + c] = val;
+                else static_cast<T*>(p.o)[off + c] = from_float<T>(val);
+            }
+        }
     }
 }
 

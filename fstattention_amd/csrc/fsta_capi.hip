@@ -116,6 +116,10 @@ extern "C" int fsta_attention_fwd_ws(const void* q, const void* k, const void* v
     if (slices == 0 || nq == 0) return FSTA_OK;
     if (!q || !k || !v || !o || !ancestor_idx || !mask_bits || !leaf_idx)
         return fail(FSTA_EINVAL, "fsta_attention_fwd: null pointer");
+    // rows are moved 16 bytes at a time
+    if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+         reinterpret_cast<uintptr_t>(o)) % 16 != 0)
+        return fail(FSTA_EINVAL, "fsta_attention_fwd: q, k, v and o must be 16-byte aligned");
 
     AttnParams p;
     p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse;

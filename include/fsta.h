@@ -120,6 +120,7 @@ int fsta_pack_mask(const int64_t* ancestor_idx, const uint8_t* ancestor_mask,
  * num_blocks must equal ceil(nq / block_m).  A row that attends to nothing
  * gets o = 0 and lse = -inf.
  * head_dim in {16,32,64,128}; block_m in {16,32,64,128}; max_ancestors >= 1.
+ * q, k, v and o must be 16-byte aligned (rows are moved 16 bytes at a time).
  */
 int fsta_attention_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                        const int64_t* ancestor_idx, const uint32_t* mask_bits,
