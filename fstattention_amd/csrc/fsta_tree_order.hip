@@ -219,10 +219,34 @@ __global__ __launch_bounds__(kSmallThreads) void order_small_kernel(const int64_
     }
 }
 
+// new_parent[rank[i]] = rank[parent[i]]: the same forest with node i renamed rank[i]
+__global__ __launch_bounds__(kOrderThreads) void renumber_kernel(const int64_t* __restrict__ parent,
+                                                                 const int64_t* __restrict__ rank, int64_t n,
+                                                                 int64_t* __restrict__ new_parent) {
+    const int64_t i = (int64_t)blockIdx.x * kOrderThreads + threadIdx.x;
+    if (i >= n) return;
+    const int64_t p = parent[i], r = rank[i];
+    if (r < 0 || r >= n) return;                      // not a permutation: nothing written for this node
+    new_parent[r] = (p >= 0 && p < n) ? rank[p] : -1;
+}
+
 }  // namespace
 }  // namespace fsta
 
 using namespace fsta;
+
+extern "C" int fsta_renumber_parents(const int64_t* parent, const int64_t* rank, int64_t n_nodes,
+                                     int64_t* new_parent, void* stream) {
+    if (n_nodes < 0) return fail(FSTA_EINVAL, "fsta_renumber_parents: n_nodes=%lld", (long long)n_nodes);
+    if (n_nodes == 0) return FSTA_OK;
+    if (!parent || !rank || !new_parent) return fail(FSTA_EINVAL, "fsta_renumber_parents: null pointer");
+    const int64_t blocks = (n_nodes + kOrderThreads - 1) / kOrderThreads;
+    if (blocks > 0x7fffffff) return fail(FSTA_EUNSUPPORTED, "fsta_renumber_parents: n_nodes=%lld", (long long)n_nodes);
+    hipLaunchKernelGGL(renumber_kernel, dim3((unsigned)blocks), dim3(kOrderThreads), 0, static_cast<hipStream_t>(stream),
+                       parent, rank, n_nodes, new_parent);
+    FSTA_HIP_OK(hipGetLastError());
+    return FSTA_OK;
+}
 
 extern "C" int fsta_dfs_order(const int64_t* parent, int64_t n_nodes, int32_t light_first, int64_t* perm,
                               int64_t* rank, int32_t* workspace, uint32_t* status, void* stream) {

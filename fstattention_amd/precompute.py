@@ -26,7 +26,7 @@ def _raise_for_status(status: int, max_ancestors: int):
 
 def create_fst_attention_kernel_inputs(lineage, level_lookup, block_m=64, max_ancestors=32, *,
                                        mutate_lineage: bool = True, check: bool = True,
-                                       want_bool_mask: bool = True, device=None):
+                                       want_bool_mask: bool = True, device=None, status=None):
     """``(ancestor_idx, ancestor_mask, leaf_idx)`` of reference ``utils.py:104-129``.
 
     ``ancestor_idx`` int64 ``[NB, max_ancestors]`` (ascending, ``-1`` padded),
@@ -40,7 +40,9 @@ def create_fst_attention_kernel_inputs(lineage, level_lookup, block_m=64, max_an
     ``RuntimeError`` when a block has more than ``max_ancestors`` ancestors;
     with ``check=False`` a 4th value, the device status word, is returned
     instead.  ``want_bool_mask=False`` returns a :class:`PackedTreeMask` in
-    place of the bool tensor.
+    place of the bool tensor.  ``status``: a zeroed int32 ``[1]`` tensor on the device to
+    collect the status bits in (the stages of a front-end chain can share one, which spares
+    each of them the fill of its own).
     """
     if lineage.dim() != 2 or level_lookup.dim() != 1 or level_lookup.shape[0] != lineage.shape[0]:
         raise ValueError(f"lineage {tuple(lineage.shape)} / level_lookup {tuple(level_lookup.shape)}")
@@ -67,7 +69,8 @@ def create_fst_attention_kernel_inputs(lineage, level_lookup, block_m=64, max_an
     l_idx = torch.empty((nb, block_m), dtype=torch.int64, device=dev)
     bits = torch.empty((nb, words, block_m), dtype=torch.int32, device=dev)
     count = torch.empty((nb,), dtype=torch.int32, device=dev)
-    status = torch.zeros((1,), dtype=torch.int32, device=dev)
+    if status is None:
+        status = torch.zeros((1,), dtype=torch.int32, device=dev)
     with _on_device(dev):
         _lib.check(lib.fsta_precompute(
             lin.data_ptr(), lvl.data_ptr(), n, width, block_m, max_ancestors, int(mutate_lineage),
@@ -88,11 +91,12 @@ def create_fst_attention_kernel_inputs(lineage, level_lookup, block_m=64, max_an
     return out if check else out + (status,)
 
 
-def lineage_from_parents_gpu(parent: torch.Tensor, width: Optional[int] = None, check: bool = True):
+def lineage_from_parents_gpu(parent: torch.Tensor, width: Optional[int] = None, check: bool = True, status=None):
     """``parent [N]`` int64 on the GPU -> ``(lineage [N, width], level_lookup [N])`` on the GPU.
 
     Layout of reference ``utils.py:66-75``.  Without ``width`` the levels are
     computed first and ``max(level) + 1`` is read back (one synchronisation).
+    ``status``: optional zeroed int32 ``[1]`` device tensor to collect the status bits in.
     """
     if not parent.is_cuda or parent.dtype != torch.int64 or parent.dim() != 1:
         raise ValueError("parent must be a 1-D int64 tensor on the GPU")
@@ -101,7 +105,8 @@ def lineage_from_parents_gpu(parent: torch.Tensor, width: Optional[int] = None, 
     dev = parent.device
     n = parent.shape[0]
     level = torch.empty((n,), dtype=torch.int64, device=dev)
-    status = torch.zeros((1,), dtype=torch.int32, device=dev)
+    if status is None:
+        status = torch.zeros((1,), dtype=torch.int32, device=dev)
     with _on_device(dev):
         if width is None:
             _lib.check(lib.fsta_lineage_from_parents(parent.data_ptr(), n, 1, None, level.data_ptr(),
@@ -119,13 +124,14 @@ def lineage_from_parents_gpu(parent: torch.Tensor, width: Optional[int] = None, 
     return lineage, level
 
 
-def dfs_order_gpu(parent: torch.Tensor, children: str = "index", check: bool = True):
+def dfs_order_gpu(parent: torch.Tensor, children: str = "index", check: bool = True, status=None):
     """``parent [N]`` int64 on the GPU -> ``(perm, rank)`` int64 ``[N]`` on the GPU.
 
     Device version of ``trees.dfs_order`` (``perm[new] = old``, ``rank[old] = new``) for trees
     that are rebuilt on the GPU every decoding step; no host synchronisation with
     ``check=False``.  ``renumber_parents_gpu`` applies the order to the tree, ``index_select``
-    to the token tensors.
+    to the token tensors.  ``status``: optional zeroed int32 ``[1]`` device tensor to collect the
+    status bits in.
     """
     if not parent.is_cuda or parent.dtype != torch.int64 or parent.dim() != 1:
         raise ValueError("parent must be a 1-D int64 tensor on the GPU")
@@ -138,7 +144,8 @@ def dfs_order_gpu(parent: torch.Tensor, children: str = "index", check: bool = T
     perm = torch.empty((n,), dtype=torch.int64, device=dev)
     rank = torch.empty((n,), dtype=torch.int64, device=dev)
     work = torch.empty((2 * n,), dtype=torch.int32, device=dev)
-    status = torch.zeros((1,), dtype=torch.int32, device=dev)
+    if status is None:
+        status = torch.zeros((1,), dtype=torch.int32, device=dev)
     with _on_device(dev):
         _lib.check(lib.fsta_dfs_order(parent.data_ptr(), n, 1 if children == "light_first" else 0,
                                       perm.data_ptr(), rank.data_ptr(), work.data_ptr(),
@@ -149,12 +156,20 @@ def dfs_order_gpu(parent: torch.Tensor, children: str = "index", check: bool = T
 
 
 def renumber_parents_gpu(parent: torch.Tensor, perm: torch.Tensor, rank: torch.Tensor) -> torch.Tensor:
-    """Parent array of the same forest after node ``perm[new]`` has been renamed ``new``."""
-    old_parent = parent.index_select(0, perm)
-    return torch.where(old_parent >= 0, rank.index_select(0, old_parent.clamp(min=0)), old_parent)
+    """Parent array of the same forest after node ``perm[new]`` has been renamed ``new`` (one launch)."""
+    if not (parent.is_cuda and rank.is_cuda) or parent.dtype != torch.int64 or rank.dtype != torch.int64 or \
+            parent.shape != rank.shape or parent.dim() != 1:
+        raise ValueError("parent and rank must be 1-D int64 tensors of one length on the GPU")
+    lib = _lib.load()
+    parent, rank = parent.contiguous(), rank.contiguous()
+    new_parent = torch.empty_like(parent)
+    with _on_device(parent.device):
+        _lib.check(lib.fsta_renumber_parents(parent.data_ptr(), rank.data_ptr(), parent.shape[0],
+                                             new_parent.data_ptr(), _stream_ptr(parent.device)))
+    return new_parent
 
 
-def medusa_parents_gpu(probs: torch.Tensor, n: int, check: bool = False) -> torch.Tensor:
+def medusa_parents_gpu(probs: torch.Tensor, n: int, check: bool = False, status=None) -> torch.Tensor:
     """``probs [depths, topk]`` on the GPU -> parent array int64 ``[n]`` on the GPU, no host round trip.
 
     Device version of ``trees.medusa_parents_from_probs`` (same selection, same tie-breaks, same
@@ -166,7 +181,8 @@ def medusa_parents_gpu(probs: torch.Tensor, n: int, check: bool = False) -> torc
     tensor operations); with ``dfs_order_gpu``, ``lineage_from_parents_gpu(width=depths + 1)`` and
     ``create_fst_attention_kernel_inputs(check=False)`` a tree goes from draft-head probabilities
     to kernel inputs without touching the host.  ``check`` synchronises and raises when a kept
-    path's prefix was not kept (probabilities above 1 or not numbers).
+    path's prefix was not kept (probabilities above 1 or not numbers).  ``status``: optional zeroed
+    int32 ``[1]`` device tensor to collect the status bits in.
     """
     if probs.dim() != 2 or not probs.is_cuda:
         raise ValueError("probs must be a [depths, topk] tensor on the GPU")
@@ -182,7 +198,8 @@ def medusa_parents_gpu(probs: torch.Tensor, n: int, check: bool = False) -> torc
     lib = _lib.load()
     dev = probs.device
     parent = torch.empty((n,), dtype=torch.int64, device=dev)
-    status = torch.zeros((1,), dtype=torch.int32, device=dev)
+    if status is None:
+        status = torch.zeros((1,), dtype=torch.int32, device=dev)
     with _on_device(dev):
         _lib.check(lib.fsta_medusa_tree(probs.data_ptr(), _lib.F32 if probs.dtype == torch.float32 else _lib.F64,
                                         depths, topk, n, parent.data_ptr(), status.data_ptr(), _stream_ptr(dev)))

@@ -205,6 +205,15 @@ int fsta_merge_states(const void* o_a, const float* lse_a, const void* o_b, cons
                       void* stream);
 
 /*
+ * new_parent[rank[i]] = rank[parent[i]] (-1 for roots): the parent array of the same
+ * forest after node i has been renamed rank[i], e.g. with the rank of
+ * fsta_dfs_order.  No counterpart in the reference (see fsta_dfs_order).  rank must
+ * be a permutation of 0 .. n_nodes-1; new_parent must not alias parent.
+ */
+int fsta_renumber_parents(const int64_t* parent, const int64_t* rank, int64_t n_nodes,
+                          int64_t* new_parent, void* stream);
+
+/*
  * Draft-head probabilities -> parent array of the tree of the most probable candidate
  * paths (a Medusa-style static tree), on the device.  No counterpart in the reference,
  * which builds its trees on the host (utils.py:27-77); with fsta_dfs_order,

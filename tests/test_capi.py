@@ -74,6 +74,9 @@ def test_argument_validation_happens_before_any_gpu_work():
     assert lib.fsta_dfs_order(None, -1, 0, None, None, None, None, None) == _lib.EINVAL
     assert lib.fsta_dfs_order(None, 1 << 20, 0, None, None, None, None, None) == _lib.EUNSUPPORTED
     assert lib.fsta_dfs_order(None, 8, 0, None, None, None, None, None) == _lib.EINVAL      # null pointers
+    assert lib.fsta_renumber_parents(None, None, -1, None, None) == _lib.EINVAL
+    assert lib.fsta_renumber_parents(None, None, 0, None, None) == _lib.OK
+    assert lib.fsta_renumber_parents(None, None, 8, None, None) == _lib.EINVAL and b"null" in lib.fsta_last_error()
     assert lib.fsta_merge_states(None, None, None, None, None, None, 4, 12, _lib.BF16, None) == _lib.EINVAL   # head dim
     assert lib.fsta_merge_states(None, None, None, None, None, None, 4, 64, 7, None) == _lib.EINVAL          # null pointers come first
     assert lib.fsta_merge_states(None, None, None, None, None, None, 0, 64, _lib.BF16, None) == _lib.OK       # nothing to do

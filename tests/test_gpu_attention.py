@@ -534,12 +534,13 @@ def test_decoding_step_from_probabilities_in_one_graph():
     q, k, v = (t.cuda() for t in rand_qkv(1, 2, n, n, d, torch.bfloat16, 50))
 
     def step():
-        parent = medusa_parents_gpu(probs, n)
-        perm, rank = dfs_order_gpu(parent, "light_first", check=False)
+        status = torch.zeros((1,), dtype=torch.int32, device="cuda")      # one status word for the whole chain
+        parent = medusa_parents_gpu(probs, n, status=status)
+        perm, rank = dfs_order_gpu(parent, "light_first", check=False, status=status)
         new_parent = renumber_parents_gpu(parent, perm, rank)
-        lineage, level = lineage_from_parents_gpu(new_parent, width=depths + 1, check=False)
+        lineage, level = lineage_from_parents_gpu(new_parent, width=depths + 1, check=False, status=status)
         *inputs, status = create_fst_attention_kernel_inputs(lineage, level, m, max_anc, check=False,
-                                                             want_bool_mask=False)
+                                                             want_bool_mask=False, status=status)
         # tokens arrive in the builder's numbering: into depth-first order and back around the op
         o = fst_attention(q.index_select(2, perm), k.index_select(2, perm), v.index_select(2, perm), *inputs,
                           scale, BLOCK_M=m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32)
