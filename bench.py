@@ -301,6 +301,47 @@ def time_front_end(index, reps=20, stages=None):
     return {name: device_us(fn) for name, fn in calls.items() if stages is None or name in stages}
 
 
+def time_decoding_step(wl, layers=32, reps=5):
+    """One decoding step of the headline workload as one HIP graph: draft probabilities -> tree ->
+    depth-first order -> lineage -> kernel inputs (once), then `layers` attention calls on rotating
+    q/k/v/o sets that all use those inputs.  Microseconds per step from HIP events."""
+    import torch
+    from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, fst_attention,
+                                  lineage_from_parents_gpu, medusa_parents_gpu, renumber_parents_gpu, trees)
+    dev = torch.device("cuda", 0)
+    probs = torch.from_numpy(trees.medusa_probs()).to(dev)
+    depths = probs.shape[0]
+
+    def step():
+        status = torch.zeros((1,), dtype=torch.int32, device=dev)
+        parent = medusa_parents_gpu(probs, wl.n, status=status)
+        perm, rank = dfs_order_gpu(parent, "light_first", check=False, status=status)
+        new_parent = renumber_parents_gpu(parent, perm, rank)
+        lineage, level = lineage_from_parents_gpu(new_parent, width=depths + 1, check=False, status=status)
+        a_idx, packed, l_idx, _ = create_fst_attention_kernel_inputs(
+            lineage, level, wl.m, wl.max_anc, check=False, want_bool_mask=False, status=status)
+        for layer in range(layers):
+            q, k, v, _ = wl.sets[layer % wl.n_sets]
+            fst_attention(q, k, v, a_idx, packed, l_idx, wl.scale, BLOCK_M=wl.m, MAX_ANCESTORS=wl.max_anc)
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        step()
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            step()
+        graph.replay()
+        stream.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record(stream)
+        for _ in range(reps):
+            graph.replay()
+        ev1.record(stream)
+        torch.cuda.synchronize()
+    return ev0.elapsed_time(ev1) * 1e3 / reps
+
+
 def cpu_baseline(wl, budget_s=10.0):
     """The oracle's dense-masked attention (reference fstattention.py:214-219 restated for
     the CPU, float32 arithmetic on the bf16-rounded inputs) on the host cores."""
@@ -527,6 +568,12 @@ def main():
             }
             del w
             torch.cuda.empty_cache()
+        step_us = time_decoding_step(wl)
+        extra["cfg2_decoding_step"] = {
+            "layers": 32, "total_us": round(step_us, 1),
+            "note": "one graph: probabilities -> tree -> depth-first order -> lineage -> kernel inputs, then 32 "
+                    "attention calls (Python wrapper, output allocated per call) on rotating q/k/v sets",
+        }
         # the integer kernels that turn a new tree into kernel inputs once per decoding step
         extra["front_end_device_us"] = {trees_name: time_front_end(idx) for idx, trees_name in
                                         ((2, "cfg2_medusa256"), (3, "cfg3_deep1024"), (4, "cfg4_wide4096"),
