@@ -491,7 +491,7 @@ def main():
         "roofline": {
             "bound": "hbm",
             "kernel": ("attn_generic_kernel" if wl.dtype == torch.float32 else
-                       "attn_mfma16_kernel<bf16, D=128, 32-row halves of the 64-row blocks, split P, 2 key shares>"
+                       "attn_mfma16_kernel<bf16, D=128, 32-row halves of the 64-row blocks, split P, wave pairs by head-dim halves>"
                        if args.config == 2 and wl.dtype == torch.bfloat16 else "attn_mfma16_kernel"),
             "achieved": round(achieved, 2),
             "peak": HBM_PEAK_GBPS,

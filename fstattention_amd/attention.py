@@ -105,7 +105,7 @@ def _packed_for(ancestor_idx: torch.Tensor, ancestor_mask) -> PackedTreeMask:
 def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
                   BLOCK_M=128, MAX_ANCESTORS=64, *, out_dtype: Optional[torch.dtype] = None,
                   return_lse: bool = False, fast_pv: bool = False, generic: bool = False,
-                  wide_waves: bool = False, key_splits: Optional[int] = None):
+                  wide_waves: bool = False, key_splits: Optional[int] = None, share_tiles: bool = False):
     """Fused sparse tree attention forward (reference ``fstattention.py:153-181``).
 
     ``q [Z,H,Nq,D]``, ``k,v [Z,H,Nk,D]`` (``Nk - Nq`` leading rows are a dense
@@ -122,7 +122,9 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
     with 32 instead of 16 query rows per wave.  A long shared prefix in front of few
     query blocks is cut into runs of keys that separate workgroups take (the partial
     results live in a temporary workspace and are joined by a second kernel);
-    ``key_splits`` forces the number of runs (``1``: never split).  Inputs the reference silently
+    ``key_splits`` forces the number of runs (``1``: never split); ``share_tiles`` is a tuning
+    switch (wave pairs of a row group take alternate key tiles even where the library would let
+    them share the head dimension).  Inputs the reference silently
     mis-handles raise ``ValueError`` here (non-contiguous tensors, index
     tensors whose shapes do not match ``BLOCK_M`` / ``MAX_ANCESTORS``).
     """
@@ -174,7 +176,8 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
     # the reference allocates L and drops it (fstattention.py:158-160,181); here it only exists when asked for
     lse = torch.empty((Z * H, Nq), device=q.device, dtype=torch.float32) if return_lse else None
     flags = (_lib.FLAG_FAST_PV if fast_pv else 0) | (_lib.FLAG_GENERIC if generic else 0) | \
-        (_lib.FLAG_WIDE_WAVES if wide_waves else 0) | (_lib.flag_key_splits(key_splits) if key_splits else 0)
+        (_lib.FLAG_WIDE_WAVES if wide_waves else 0) | (_lib.flag_key_splits(key_splits) if key_splits else 0) | \
+        (_lib.FLAG_SHARE_TILES if share_tiles else 0)
     # a shared prefix may be worth cutting into key runs: the library says how much workspace that takes
     work, work_bytes = None, 0
     if Nk > Nq:

@@ -64,20 +64,27 @@ __device__ __forceinline__ void flush_rows(const unsigned char* stage, int strid
     }
 }
 
-// KS = waves that share one group of 16 query rows, each taking every KS-th tile with its own
-// running softmax (merged through LDS at the end).
+// KS > 0: waves that share one group of 16 query rows, each taking every KS-th tile with its own
+// running softmax (merged through LDS at the end).  KS = -2: two waves share a group of rows by
+// the head dimension instead: both walk every tile and form the same weights, each accumulates
+// and stores its half of O.  Nothing is exchanged or merged at the end, which shortens the chain
+// of a launch with one or two ancestor tiles per block; the duplicated S and softmax work makes
+// it the wrong choice for long tile lists.
 // RUNS = the launch cuts the shared prefix into runs of keys (AttnParams::key_splits > 1).
 template <bool BF16, int D, int M, bool SPLIT, int KS, bool RUNS>
-__global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p, int stages, int early_leaf, int sub_shift) {
+__global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_kernel(AttnParams p, int stages, int early_leaf, int sub_shift) {
     using MM = Mma<BF16>;
     using T = typename MM::elem;
     using T2 = typename MM::elem2;
     using Frag = typename MM::frag;
     constexpr int kQGroups = M / 16;              // groups of 16 query rows
     constexpr int kLeafTiles = M / 32;            // 32-row tiles holding the block's own rows
-    constexpr int kSplit = KS;
+    constexpr bool kDShare = KS < 0;              // the waves of a row group share the head dimension
+    constexpr int kSplit = kDShare ? 1 : KS;      // tiles per step, dealt to the waves of a row group
+    constexpr int kShares = kDShare ? -KS : KS;   // waves per row group
+    static_assert(!kDShare || (KS == -2 && D >= 64), "head-dimension halves need two accumulator tiles each");
     constexpr int kLeafGroup = leaf_group16_for(M);
-    constexpr int kWaves = kQGroups * kSplit;
+    constexpr int kWaves = kQGroups * kShares;
     constexpr int kThreads = kWaves * 64;
     constexpr int kCpr = D / 8;                   // 16-byte chunks per row
     constexpr int kRowsPerDma = 64 / kCpr;        // rows one wave-wide 1 KiB transfer covers
@@ -88,6 +95,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     constexpr int kRowGroups = (kDmaPerWave + 1) / 2;   // row groups a wave touches per tile
     constexpr int kSteps = D / 32;                // MFMAs per 16-key half of S^T
     constexpr int kDTiles = D / 16;               // 16-row tiles of O^T
+    constexpr int kOTiles = kDShare ? kDTiles / 2 : kDTiles;   // ... of which a wave accumulates these
     constexpr int kTileElems = kTileN * D;
     // Largest sum of a lane's 8 weights accepted without looking at the row maximum: far from
     // float overflow in l and O, and every single weight still converts to the 16-bit type.
@@ -128,7 +136,8 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int qgroup = wave % kQGroups;   // which 16 query rows
-    const int split = wave / kQGroups;    // which share of the tiles
+    const int split = wave / kQGroups;    // which share of the tiles (of the head dimension)
+    const int dt0 = kDShare ? split * kOTiles : 0;   // first accumulator tile of this wave
     const int lane = tid & 63;
     const int ql = lane & 15;        // query (column of S^T / O^T) of this lane
     const int g = lane >> 4;         // which quarter of the rows of an accumulator tile
@@ -392,9 +401,9 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     if (early_leaf) read_q(issued);
 
     float m_i = -INFINITY, l_i = 0.f;
-    f32x4 o[kDTiles];
+    f32x4 o[kOTiles];
 #pragma unroll
-    for (int dt = 0; dt < kDTiles; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int dt = 0; dt < kOTiles; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // Leaf tile i = the block's own rows 32i .. 32i+31 (reference fstattention.py:86-91,104-107):
     // query r sees exactly row r of it.  The two waves owning those rows take one dot product
@@ -402,20 +411,20 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     for (int base = tree ? 0 : kLeafTiles; base < kLeafTiles; base += kLeafGroup) {
         begin_step(kLeafGroup);
         const int my_tile = qgroup >> 1;
-        if (split == 0 && my_tile >= base && my_tile < base + kLeafGroup && __ballot(leaf_ok) != 0ull) {
+        if ((kDShare || split == 0) && my_tile >= base && my_tile < base + kLeafGroup && __ballot(leaf_ok) != 0ull) {
             const T* kt = tile_ptr(my_tile - base);
             const T* vt = kt + kTileElems;
             const int row = (qgroup & 1) * 16 + ql;   // this query's row of the leaf tile
             float part[2] = {0.f, 0.f};
-            u32x2 vraw[kDTiles];   // the row's V values are requested together with its K values
+            u32x2 vraw[kOTiles];   // the row's V values are requested together with its K values
             {
                 u32x4 kraw[kSteps];
 #pragma unroll
                 for (int ks = 0; ks < kSteps; ++ks)
                     kraw[ks] = lds_read_b128(lds_addr(kt + row * D + k_chunk<D>(row, 4 * ks + g) * 8));
 #pragma unroll
-                for (int dt = 0; dt < kDTiles; ++dt)   // accumulator rows 4g .. 4g+3 of tile dt: 4 head dims
-                    vraw[dt] = lds_read_b64(lds_addr(vt + row * D + k_chunk<D>(row, 2 * dt + (g >> 1)) * 8 + 4 * (g & 1)));
+                for (int dt = 0; dt < kOTiles; ++dt)   // accumulator rows 4g .. 4g+3 of tile dt0 + dt: 4 head dims
+                    vraw[dt] = lds_read_b64(lds_addr(vt + row * D + k_chunk<D>(row, 2 * (dt0 + dt) + (g >> 1)) * 8 + 4 * (g & 1)));
                 lds_wait();
 #pragma unroll
                 for (int ks = 0; ks < kSteps; ++ks) {
@@ -431,12 +440,12 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
             }
             const float dot = sum_quarters(part[0] + part[1]);
 #pragma unroll
-            for (int dt = 0; dt < kDTiles; ++dt) lds_tie(vraw[dt]);
+            for (int dt = 0; dt < kOTiles; ++dt) lds_tie(vraw[dt]);
             if (leaf_ok) {
                 m_i = dot * p.scale_log2e;
                 l_i = g == 0 ? 1.f : 0.f;
 #pragma unroll
-                for (int dt = 0; dt < kDTiles; ++dt) {
+                for (int dt = 0; dt < kOTiles; ++dt) {
                     o[dt][0] = MM::low(vraw[dt][0]);
                     o[dt][1] = MM::high(vraw[dt][0]);
                     o[dt][2] = MM::low(vraw[dt][1]);
@@ -461,8 +470,8 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
     const uint32_t v_lane0 = (uint32_t)(tr_r0 * D + v16_chunk<D>(tr_r0, tr_col >> 3) * 8 + (tr_col & 7)) * 2;
     while (consumed < total_tiles) {
         begin_step(kSplit);
-        const int t = consumed + split;
-        const T* kt = tile_ptr(split);
+        const int t = consumed + (kDShare ? 0 : split);
+        const T* kt = tile_ptr(kDShare ? 0 : split);
         const T* vt = kt + kTileElems;
         end_step(kSplit);
         uint32_t word = 0u;
@@ -491,7 +500,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
         // read: k-slots 8g .. 8g+3 are keys 4g .. 4g+3, k-slots 8g+4 .. 8g+7 keys 16+4g .. 16+4g+3.
         // Half of the head-dim tiles are requested now (LDS latency hides behind the softmax),
         // the other half behind the first MFMAs.
-        constexpr int kHalf = kDTiles / 2;
+        constexpr int kHalf = kOTiles / 2;
         const uint32_t v_addr0 = lds_addr(vt) + v_lane0;
         auto read_v = [&](VPair (&f)[kHalf], int first_dt) {
 #pragma unroll
@@ -507,7 +516,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
             for (int i = 0; i < kHalf; ++i) { lds_tie(f[i].a); lds_tie(f[i].b); }
         };
         VPair v0[kHalf], v1[kHalf];
-        read_v(v0, 0);
+        read_v(v0, dt0);
         // mask + online softmax; register j of half `sub` is key 16*sub + 4g + j.  The scale rides
         // in the FMA under the exp2.
         const uint32_t wsh = word >> (4 * g);
@@ -547,7 +556,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
             if (raise) m_i = mx;
             l_i *= alpha;
 #pragma unroll
-            for (int dt = 0; dt < kDTiles; ++dt)
+            for (int dt = 0; dt < kOTiles; ++dt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
             const float neg_m = m_i == -INFINITY ? 0.f : -m_i;
@@ -573,7 +582,7 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
         if (SPLIT) pl = __builtin_bit_cast(Frag, lo4);
         // O^T += V_tile^T . P^T
         tie_v(v0);
-        read_v(v1, kHalf);
+        read_v(v1, dt0 + kHalf);
 #pragma unroll
         for (int i = 0; i < kHalf; ++i) o[i] = mfma16(__builtin_bit_cast(Frag, v0[i]), ph, o[i]);
         if (SPLIT) {
@@ -644,7 +653,10 @@ __global__ __launch_bounds__(M * 4 * KS, 4) void attn_mfma16_kernel(AttnParams p
                                         rows_valid);
         }
     };
-    if constexpr (kSplit == 1) {
+    if constexpr (kDShare) {
+        __syncthreads();   // every wave is done with the last tile
+        finish(o, split * (D / 2), smem + (size_t)wave * 16 * kStageStride, split == 0);
+    } else if constexpr (kSplit == 1) {
         __syncthreads();   // every wave is done with the last tile
         finish(o, 0, smem + (size_t)qgroup * 16 * kStageStride, true);
     } else {
@@ -699,14 +711,15 @@ int launch_ks(const AttnParams& p, int sub_shift, hipStream_t stream) {
     while (lds > 160 * 1024 && stages > 2) lds = mfma16_lds_bytes<D, M>(p.max_anc, --stages);
     // the kernel's start-up parks Q in the last ring slots and requests up to two leaf tiles
     // into the first ones; ancestor lists too long to leave that much LDS go to the other kernel
-    constexpr int kWaves = M / 16 * KS, kQSlots = (kWaves * 16 + 2 * kTileN - 1) / (2 * kTileN);
+    constexpr int kShares = KS < 0 ? -KS : KS;
+    constexpr int kWaves = M / 16 * kShares, kQSlots = (kWaves * 16 + 2 * kTileN - 1) / (2 * kTileN);
     if (stages < kQSlots + (M / 32 < 2 ? M / 32 : 2)) {
         if (p.key_splits > 1) return FSTA_EUNSUPPORTED;   // the caller falls back to a launch without key splits
         return launch_attention_mfma(p, BF16 ? FSTA_BF16 : FSTA_F16, D, BF16 && !SPLIT, stream);
     }
     // the epilogue reuses the front of the segment: exchange area of a key split, row staging
     constexpr size_t kEpilogueBytes = KS > 1 ? (size_t)(M / 16) * 2 * ((2 + D / 8) * 256 + 16 * (D * 2 + 16))
-                                             : (size_t)M * (D * 2 + 16);
+                                             : (size_t)kWaves * 16 * (D * 2 + 16);
     if (lds < kEpilogueBytes) lds = kEpilogueBytes;
     if (lds > 160 * 1024)
         return fail(FSTA_EUNSUPPORTED, "max_ancestors=%d needs %zu bytes of LDS (limit 163840)", p.max_anc, lds);
@@ -717,18 +730,22 @@ int launch_ks(const AttnParams& p, int sub_shift, hipStream_t stream) {
     const int early = grid <= kCus && p.key_splits == 1 && lds + kQBytes <= 160 * 1024 ? 1 : 0;
     if (early) lds += kQBytes;
     if (p.key_splits > 1) {
-        if (lds > 64 * 1024) {
-            const int rc = allow_full_lds<&attn_mfma16_kernel<BF16, D, M, SPLIT, KS, true>>();
-            if (rc != FSTA_OK) return rc;
+        if constexpr (KS > 0) {
+            if (lds > 64 * 1024) {
+                const int rc = allow_full_lds<&attn_mfma16_kernel<BF16, D, M, SPLIT, KS, true>>();
+                if (rc != FSTA_OK) return rc;
+            }
+            hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT, KS, true>), dim3(grid), dim3(M * 4 * kShares),
+                               lds, stream, p, stages, early, sub_shift);
+        } else {
+            return FSTA_EUNSUPPORTED;   // (key runs are never combined with head-dimension shares)
         }
-        hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT, KS, true>), dim3(grid), dim3(M * 4 * KS), lds,
-                           stream, p, stages, early, sub_shift);
     } else {
         if (lds > 64 * 1024) {
             const int rc = allow_full_lds<&attn_mfma16_kernel<BF16, D, M, SPLIT, KS, false>>();
             if (rc != FSTA_OK) return rc;
         }
-        hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT, KS, false>), dim3(grid), dim3(M * 4 * KS), lds,
+        hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT, KS, false>), dim3(grid), dim3(M * 4 * kShares), lds,
                            stream, p, stages, early, sub_shift);
     }
     FSTA_HIP_OK(hipGetLastError());
@@ -741,6 +758,16 @@ int launch_one(const AttnParams& p, int sub_shift, hipStream_t stream) {
     // its own and the block is small (few waves); blocks of 128 rows fill the workgroup anyway.
     const int work_tiles = anc_tile_capacity(p.max_anc) + (p.prefix + kTileN - 1) / kTileN;
     if constexpr (M < 128) {
+        if constexpr (D >= 64) {
+            // One or two ancestor tiles, no prefix, and a launch whose workgroups all run at once (its
+            // time is the length of one workgroup's chain): the two waves of a row group share the
+            // head dimension, with no exchange at the end, instead of the tiles.  With several rounds
+            // of workgroups the duplicated work costs more than the shorter chain gains (cfg4: +50 %).
+            const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
+            const bool one_round = kXcds * slices_per_xcd * (p.nb << sub_shift) <= kCus;
+            if (one_round && work_tiles <= 2 && p.prefix == 0 && p.key_splits == 1 && !p.share_tiles)
+                return launch_ks<BF16, D, M, SPLIT, -2>(p, sub_shift, stream);
+        }
         if (work_tiles >= 2) return launch_ks<BF16, D, M, SPLIT, 2>(p, sub_shift, stream);
     }
     return launch_ks<BF16, D, M, SPLIT, 1>(p, sub_shift, stream);

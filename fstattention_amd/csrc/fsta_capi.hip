@@ -132,6 +132,7 @@ extern "C" int fsta_attention_fwd_ws(const void* q, const void* k, const void* v
     p.out_f32 = (out_dtype == FSTA_F32) ? 1 : 0;
     p.scale_log2e = sm_scale * kLog2e;
     p.key_splits = 1; p.split_tiles = 0; p.part_o = nullptr; p.part_lse = nullptr;
+    p.share_tiles = (flags & FSTA_FLAG_SHARE_TILES) ? 1 : 0;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (workspace) {

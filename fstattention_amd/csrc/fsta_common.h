@@ -32,6 +32,7 @@ struct AttnParams {
     // block takes prefix tiles [s * split_tiles, (s + 1) * split_tiles) and writes a normalised
     // float32 partial result part_o[s][batch*heads][nq][D] with log-sum-exp part_lse[s][batch*heads][nq].
     int32_t key_splits, split_tiles;
+    int32_t share_tiles;          // tuning: wave pairs of a row group always share the tiles, never the head dimension
     float* part_o;
     float* part_lse;
 };

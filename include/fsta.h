@@ -44,6 +44,9 @@ extern "C" {
                                   (32x32x16 MFMA, 2 waves per SIMD) instead of 16
                                   rows per wave (16x16x32 MFMA, 4 waves per SIMD) */
 
+#define FSTA_FLAG_SHARE_TILES 8u /* tuning: where two waves share a group of 16 query rows they
+                                  always take alternate key tiles (and merge at the end), never
+                                  halves of the head dimension                              */
 #define FSTA_FLAG_KEY_SPLITS(n) (((uint32_t)(n) & 0xffu) << 8)
                                /* fsta_attention_fwd_ws / fsta_attention_workspace_bytes:
                                   cut the shared prefix into n runs of keys (n = 1: never

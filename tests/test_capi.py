@@ -40,8 +40,9 @@ def test_constants_match_header():
     assert int(defs["FSTA_TREE_NOT_PREFIX_CLOSED"]) == _lib.TREE_NOT_PREFIX_CLOSED
     assert (int(defs["FSTA_OK"]), int(defs["FSTA_EINVAL"]), int(defs["FSTA_EUNSUPPORTED"]),
             int(defs["FSTA_EHIP"])) == (_lib.OK, _lib.EINVAL, _lib.EUNSUPPORTED, _lib.EHIP)
-    assert (int(defs["FSTA_FLAG_FAST_PV"]), int(defs["FSTA_FLAG_GENERIC"]), int(defs["FSTA_FLAG_WIDE_WAVES"])) == \
-        (_lib.FLAG_FAST_PV, _lib.FLAG_GENERIC, _lib.FLAG_WIDE_WAVES)
+    assert (int(defs["FSTA_FLAG_FAST_PV"]), int(defs["FSTA_FLAG_GENERIC"]), int(defs["FSTA_FLAG_WIDE_WAVES"]),
+            int(defs["FSTA_FLAG_SHARE_TILES"])) == \
+        (_lib.FLAG_FAST_PV, _lib.FLAG_GENERIC, _lib.FLAG_WIDE_WAVES, _lib.FLAG_SHARE_TILES)
     assert (int(defs["FSTA_PRE_TOO_MANY_ANCESTORS"]), int(defs["FSTA_PRE_BAD_NODE_ID"]),
             int(defs["FSTA_PRE_BAD_LEVEL"])) == (_lib.PRE_TOO_MANY_ANCESTORS, _lib.PRE_BAD_NODE_ID, _lib.PRE_BAD_LEVEL)
 

@@ -20,7 +20,7 @@ pytestmark = pytest.mark.gpu
 
 
 def run_tree(parent, block_m, z, h, d, dtype, seed, prefix=0, generic=False, fast_pv=False,
-             scale=None, check_lse=True, wide_waves=False, key_splits=None):
+             scale=None, check_lse=True, wide_waves=False, key_splits=None, share_tiles=False):
     n = len(parent)
     a_idx, a_mask, l_idx, max_anc = oracle_inputs(parent, block_m)
     nb = a_idx.shape[0]
@@ -33,7 +33,7 @@ def run_tree(parent, block_m, z, h, d, dtype, seed, prefix=0, generic=False, fas
     o, lse = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(),
                            scale, BLOCK_M=block_m, MAX_ANCESTORS=max_anc,
                            out_dtype=torch.float32, return_lse=True, generic=generic, fast_pv=fast_pv,
-                           wide_waves=wide_waves, key_splits=key_splits)
+                           wide_waves=wide_waves, key_splits=key_splits, share_tiles=share_tiles)
     assert o.dtype == torch.float32 and o.shape == q.shape
     err = assert_close(o, want, dtype, f"n={n} m={block_m} d={d} {dtype} prefix={prefix}")
     if check_lse:
@@ -220,6 +220,19 @@ def test_key_runs_native_output_type_and_workspace_contract():
                             out_dtype=torch.float32, key_splits=1)
     assert torch.equal(outs[0], unsplit) and torch.equal(outs[1], unsplit)
     assert not torch.equal(outs[2], unsplit)      # the split path did run
+
+
+@pytest.mark.parametrize("share_tiles", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("block_m,d", [(32, 64), (32, 128), (64, 64), (64, 128), (128, 128), (128, 64)])
+def test_short_ancestor_lists_both_wave_pairings(block_m, d, dtype, share_tiles):
+    """Small launches with one or two ancestor tiles per block: the waves of a row group share the
+    head dimension by default and the key tiles with the tuning flag; ragged last block included."""
+    parent = trees.medusa_parents(n=230, seed=500 + d + block_m)
+    run_tree(parent, block_m, 1, 5, d, dtype, 17, share_tiles=share_tiles)
+    bushy = np.maximum((np.arange(90) - 1) // 3, -1).astype(np.int64)      # at most one ancestor tile
+    bushy[0] = -1
+    run_tree(bushy, block_m, 2, 2, d, dtype, 18, share_tiles=share_tiles)
 
 
 def test_reference_test_shape_with_and_without_prefix():
