@@ -759,13 +759,14 @@ int launch_one(const AttnParams& p, int sub_shift, hipStream_t stream) {
     const int work_tiles = anc_tile_capacity(p.max_anc) + (p.prefix + kTileN - 1) / kTileN;
     if constexpr (M < 128) {
         if constexpr (D >= 64) {
-            // One or two ancestor tiles, no prefix, and a launch whose workgroups all run at once (its
+            // Up to four ancestor tiles, no prefix, and a launch whose workgroups all run at once (its
             // time is the length of one workgroup's chain): the two waves of a row group share the
             // head dimension, with no exchange at the end, instead of the tiles.  With several rounds
-            // of workgroups the duplicated work costs more than the shorter chain gains (cfg4: +50 %).
+            // of workgroups the duplicated work costs more than the shorter chain gains (cfg4: +50 %),
+            // and so it does with longer lists (8 tiles: +10 %).
             const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
             const bool one_round = kXcds * slices_per_xcd * (p.nb << sub_shift) <= kCus;
-            if (one_round && work_tiles <= 2 && p.prefix == 0 && p.key_splits == 1 && !p.share_tiles)
+            if (one_round && work_tiles <= 4 && p.prefix == 0 && p.key_splits == 1 && !p.share_tiles)
                 return launch_ks<BF16, D, M, SPLIT, -2>(p, sub_shift, stream);
         }
         if (work_tiles >= 2) return launch_ks<BF16, D, M, SPLIT, 2>(p, sub_shift, stream);
