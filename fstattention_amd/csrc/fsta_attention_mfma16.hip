@@ -457,9 +457,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     }
 
     // Ancestor tiles under the packed tree mask, then the dense shared prefix; kSplit tiles per
-    // step, tile consumed+s by the waves of share s.  A tile none of a wave's queries attends
-    // to is not skipped: with an all-zero mask word it adds exact zeros, and a branch-free body
-    // spares the accumulators a copy per step.
+    // step, tile consumed+s by the waves of share s.
     // Byte offsets of this lane's fragments inside a tile.  The XOR swizzles only touch the
     // chunk bits, so the fragment of K-step ks / head-dim tile dt sits at offset0 ^ (ks << 6)
     // resp. offset0 ^ (dt << 5), and the rows 16 further down at a fixed distance.
@@ -482,6 +480,10 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
             word = left >= 32 ? 0xffffffffu : ((1u << left) - 1u);
         }
         if (kSplit > 1 && t >= total_tiles) continue;   // this share has no tile in the last step
+        // A tile none of this wave's 16 queries attends to (10-30 % of the ancestor tiles of deep
+        // trees) is skipped where a workgroup walks long lists; in the short chains of the
+        // head-dimension pairing the branch costs more than the rare skip saves.
+        if (!kDShare && __ballot(word != 0u) == 0ull) continue;
 
         // S^T = K_tile . Q^T, two halves of 16 keys
         typedef const u32x4 __attribute__((address_space(3))) * lds_u32x4;
