@@ -109,6 +109,14 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     uint32_t* spec_s = valid_s + ((cap + 3) & ~3);                           // [8] per-wave flags of the start-up
     uint32_t* mask_s = spec_s + 8;                                           // [ancestor tiles][M], 16-byte aligned
 
+    // All kernel arguments are fetched by ONE batch of scalar loads.  Left to itself the compiler
+    // loads each field just before its first use, which puts four dependent round trips to the
+    // argument segment in front of the first memory request of the workgroup.
+    asm volatile("" ::"s"(p.q), "s"(p.k), "s"(p.v), "s"(p.o), "s"(p.lse), "s"(p.ancestor_idx), "s"(p.mask_bits),
+                 "s"(p.anc_count), "s"(p.leaf_idx), "s"(p.nq), "s"(p.nk), "s"(p.prefix), "s"(p.max_anc),
+                 "s"(p.mask_words), "s"(p.nb), "s"(p.heads_total), "s"(p.out_f32), "s"(p.scale_log2e), "s"(stages),
+                 "s"(early_leaf), "s"(sub_shift));
+
     // Workgroup -> (slice, block), XCD-aware: every XCD gets whole (batch, head) slices, so all
     // query blocks of a slice share one L2 for the K/V rows they have in common.
     const int xcd = blockIdx.x % kXcds;
@@ -153,7 +161,9 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     // mask words, key lists, Q rows, then the first leaf tiles.  The number of transfers issued
     // after the key lists is a compile-time constant: the wait for the lists can then leave
     // exactly those in flight.
-    int n_anc = p.anc_count ? p.anc_count[j] : p.max_anc;
+    // (the block's ancestor count: requested first, read when the key lists have arrived)
+    uint32_t anc_count_raw = 0u;
+    if (p.anc_count) anc_count_raw = global_read_b32(p.anc_count + j);
     // mask words: straight global->LDS copy, 16 bytes per lane, 1 KiB pieces dealt to the waves
     {
         // source: [word][block_rows] words of block j, of which this workgroup takes M per word
@@ -319,6 +329,8 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         }
     };
     if (!early_leaf) read_q(0);   // Q sits in ring slots the gathers are about to take
+    lds_tie(anc_count_raw);
+    int n_anc = p.anc_count ? __builtin_amdgcn_readfirstlane((int)anc_count_raw) : p.max_anc;
     n_anc = tree ? min(max(n_anc, 0), p.max_anc) : 0;
     const int listed_tiles = kLeafTiles + (n_anc + kTileN - 1) / kTileN;
     int prefix_first = 0, prefix_end = (p.prefix + kTileN - 1) / kTileN;   // this workgroup's prefix tiles

@@ -140,6 +140,11 @@ __device__ __forceinline__ u32x2 global_read_b64(const void* ptr) {
     asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(out) : "v"(ptr) : "memory");
     return out;
 }
+__device__ __forceinline__ uint32_t global_read_b32(const void* ptr) {
+    uint32_t out;
+    asm volatile("global_load_dword %0, %1, off" : "=v"(out) : "v"(ptr) : "memory");
+    return out;
+}
 // LDS store the compiler does not see either (same reason); complete after lds_wait().
 __device__ __forceinline__ void lds_write_b32(uint32_t addr, uint32_t value) {
     asm volatile("ds_write_b32 %0, %1" : : "v"(addr), "v"(value) : "memory");
