@@ -312,6 +312,7 @@ __global__ __launch_bounds__(kThreads) void lineage_from_parents_kernel(
 __global__ __launch_bounds__(kThreads) void lineage_rows_kernel(
     const int64_t* __restrict__ parent, int n, int width, int rows_per_wg,
     int64_t* __restrict__ lineage, int64_t* __restrict__ level_lookup, uint32_t* __restrict__ status) {
+    asm volatile("" ::"s"(parent), "s"(n), "s"(width), "s"(rows_per_wg), "s"(lineage), "s"(level_lookup), "s"(status));   // one batch of argument loads
     extern __shared__ int32_t rows_s[];
     int32_t* par_s = rows_s;                  // [n]
     int32_t* depth_s = par_s + n;             // [rows_per_wg], -1: the row stays empty

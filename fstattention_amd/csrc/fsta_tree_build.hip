@@ -31,6 +31,7 @@ template <typename T>
 __global__ __launch_bounds__(kBuildThreads) void medusa_tree_kernel(const T* __restrict__ probs, int depths, int topk,
                                                                     int n_cand, int keep, int64_t* __restrict__ parent,
                                                                     uint32_t* __restrict__ status) {
+    asm volatile("" ::"s"(probs), "s"(depths), "s"(topk), "s"(n_cand), "s"(keep), "s"(parent), "s"(status));   // one batch of argument loads
     extern __shared__ __attribute__((aligned(16))) unsigned char build_s[];
     uint64_t* key_s = reinterpret_cast<uint64_t*>(build_s);                    // [n_cand] score bits, later node ids
     double* prob_s = reinterpret_cast<double*>(key_s + n_cand);                // [depths * topk]

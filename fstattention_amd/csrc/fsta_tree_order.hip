@@ -141,6 +141,7 @@ __global__ __launch_bounds__(kSmallThreads) void order_small_kernel(const int64_
                                                                     int light_first, int64_t* __restrict__ perm,
                                                                     int64_t* __restrict__ rank,
                                                                     uint32_t* __restrict__ status) {
+    asm volatile("" ::"s"(parent), "s"(n), "s"(light_first), "s"(perm), "s"(rank), "s"(status));   // one batch of argument loads
     extern __shared__ int32_t small_s[];
     int32_t* par_s = small_s;          // [n]   parent, -1 for roots
     int32_t* size_s = par_s + n;       // [n]   nodes in the subtree
