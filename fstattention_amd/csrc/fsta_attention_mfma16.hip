@@ -157,29 +157,13 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     const T* vb = static_cast<const T*>(p.v) + (size_t)hz * p.nk * D;
 
     // ---- start-up: everything that needs no metadata goes out before the metadata is read ----
-    // Loads and transfers retire in issue order, so the order below is also the order of use:
-    // mask words, key lists, Q rows, then the first leaf tiles.  The number of transfers issued
-    // after the key lists is a compile-time constant: the wait for the lists can then leave
-    // exactly those in flight.
+    // Loads and transfers retire in issue order.  The key lists go first (the longest chain hangs
+    // on them: sanitise, barrier, ancestor requests), then mask words, Q rows and the first leaf
+    // tiles.  The number of transfers issued after the mask words is a compile-time constant: the
+    // wait for the lists (and the mask words behind them) can then leave exactly those in flight.
     // (the block's ancestor count: requested first, read when the key lists have arrived)
     uint32_t anc_count_raw = 0u;
     if (p.anc_count) anc_count_raw = global_read_b32(p.anc_count + j);
-    // mask words: straight global->LDS copy, 16 bytes per lane, 1 KiB pieces dealt to the waves
-    {
-        // source: [word][block_rows] words of block j, of which this workgroup takes M per word
-        const int chunks = p.mask_words * (M / 4);     // 16-byte pieces
-        const char* src = reinterpret_cast<const char*>(p.mask_bits) +
-                          ((size_t)j * p.mask_words * block_rows + (row_base - j * block_rows)) * 4;
-        for (int piece = wave; piece * 64 < chunks; piece += kWaves) {
-            const int c = piece * 64 + lane;
-            if (c < chunks)
-                __builtin_amdgcn_global_load_lds(
-                    (const void __attribute__((address_space(1)))*)(src + ((size_t)(c / (M / 4)) * block_rows * 4 +
-                                                                           (c % (M / 4)) * 16)),
-                    (void __attribute__((address_space(3)))*)(reinterpret_cast<char*>(mask_s) + piece * 1024),
-                    16, 0, 0);
-        }
-    }
     // Key lists: the block's M leaf slots, then its ancestor slots, kKeyBatch per thread and
     // round.  Slots past the end of the lists re-read the last entry and are blanked below.
     constexpr int kKeyBatch = 2;
@@ -203,6 +187,22 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     u32x2 leaf_raw = global_read_b64(p.leaf_idx + (size_t)row_base + row_in_block);
     u32x2 first_raw[kKeyBatch];
     load_ids(tid, first_raw);
+    // mask words: straight global->LDS copy, 16 bytes per lane, 1 KiB pieces dealt to the waves
+    {
+        // source: [word][block_rows] words of block j, of which this workgroup takes M per word
+        const int chunks = p.mask_words * (M / 4);     // 16-byte pieces
+        const char* src = reinterpret_cast<const char*>(p.mask_bits) +
+                          ((size_t)j * p.mask_words * block_rows + (row_base - j * block_rows)) * 4;
+        for (int piece = wave; piece * 64 < chunks; piece += kWaves) {
+            const int c = piece * 64 + lane;
+            if (c < chunks)
+                __builtin_amdgcn_global_load_lds(
+                    (const void __attribute__((address_space(1)))*)(src + ((size_t)(c / (M / 4)) * block_rows * 4 +
+                                                                           (c % (M / 4)) * 16)),
+                    (void __attribute__((address_space(3)))*)(reinterpret_cast<char*>(mask_s) + piece * 1024),
+                    16, 0, 0);
+        }
+    }
     // Q rows of this wave: whole rows straight into LDS, K-tile swizzle, parked in the last ring
     // slots until the fragments have been read (before the first barrier).  Rows past the end of
     // a ragged last block are read as the last row and never stored.
