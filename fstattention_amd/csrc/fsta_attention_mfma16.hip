@@ -368,7 +368,17 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
             issue_slot = issue_slot + 1 == stages ? 0 : issue_slot + 1;
         }
     };
+    bool all_landed = false;   // every tile of the list is in LDS and every wave knows it
     auto begin_step = [&](int n) {
+        if (kDShare && all_landed) return;
+        if (kDShare && issued == total_tiles && consumed >= kLeafTiles) {
+            // short list, the last tiles are in flight: wait for all of them once instead of
+            // passing a barrier per step
+            wait_vmcnt<0>();
+            ring_barrier();
+            all_landed = true;
+            return;
+        }
         if (issued < min(consumed + n, total_tiles)) {
             // ring too shallow (long ancestor lists leave little LDS) for this step's tiles to be
             // in flight already: free the slots first, then request them
