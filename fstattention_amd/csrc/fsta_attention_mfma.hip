@@ -70,6 +70,10 @@ __global__ __launch_bounds__(M * 2 * key_split_for(M), 2) void attn_mfma_kernel(
     constexpr int kDTiles = D / 32;               // 32-row tiles of O^T
     constexpr int kTileElems = kTileN * D;
 
+    // (all kernel arguments in one batch of scalar loads instead of one round trip per first use)
+    asm volatile("" ::"s"(p.q), "s"(p.k), "s"(p.v), "s"(p.o), "s"(p.lse), "s"(p.ancestor_idx), "s"(p.mask_bits),
+                 "s"(p.anc_count), "s"(p.leaf_idx), "s"(p.nq), "s"(p.nk), "s"(p.prefix), "s"(p.max_anc),
+                 "s"(p.mask_words), "s"(p.nb), "s"(p.heads_total), "s"(p.out_f32), "s"(p.scale_log2e), "s"(stages));
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     T* ring = reinterpret_cast<T*>(smem);                 // [stages][K tile | V tile]
     int* key_s = reinterpret_cast<int*>(ring + stages * 2 * kTileElems);
