@@ -31,7 +31,7 @@ __device__ __forceinline__ void load16(const T* src, float (&out)[Vec16<T>::n]) 
 template <int D, int M>
 constexpr size_t generic_lds_bytes() {
     return sizeof(float) * (size_t)(M * (D + kPad) + 2 * kTileN * (D + kPad) + M * (kTileN + kPad) + 2 * M)
-           + sizeof(int) * kTileN;
+           + sizeof(int) * 2 * kTileN;
 }
 
 // Register tiles: a thread owns kRowsS x 4 scores of a tile (4 neighbouring keys) and kRowsO x 4
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
     float* s_s = v_s + kTileN * kPitch;         // [M][kPitchS] scores, then weights
     float* alpha_s = s_s + M * kPitchS;         // [M] rescale of the running sums
     float* stat_s = alpha_s + M;                // [M] 1/l for the epilogue
-    int* key_s = reinterpret_cast<int*>(stat_s + M);  // [kTileN] K/V row of each tile column
+    int* key_s = reinterpret_cast<int*>(stat_s + M);  // [2][kTileN] K/V row of each tile column, tiles t and t + 1
 
     const int tid = threadIdx.x;
     const int j = blockIdx.x;
@@ -94,39 +94,72 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
     const int prefix_tiles = (p.prefix + kTileN - 1) / kTileN;
     const int total_tiles = anc_tiles + leaf_tiles + prefix_tiles;
 
+    // kind 0: ancestors, 1: leaves (diagonal), 2: shared prefix
+    auto tile_kind = [&](int t, int& base) {
+        if (t < anc_tiles) { base = t * kTileN; return 0; }
+        if (t < anc_tiles + leaf_tiles) { base = (t - anc_tiles) * kTileN; return 1; }
+        base = (t - anc_tiles - leaf_tiles) * kTileN;
+        return 2;
+    };
+    // The tile loop is a software pipeline: while tile t is worked on, the K/V rows of tile t + 1 are
+    // on their way into registers and the key list of tile t + 2 into a register of the first 32
+    // threads; each tile costs compute time only, not two dependent memory round trips as well.
+    auto load_key = [&](int t) -> int {          // threads 0 .. 31: K/V row of column tid of tile t, or -1
+        if (t >= total_tiles) return -1;
+        int base;
+        const int kind = tile_kind(t, base);
+        int64_t idx = -1;
+        const int c = base + tid;
+        if (kind == 0) { if (c < n_anc) idx = p.ancestor_idx[(size_t)j * p.max_anc + c]; }
+        else if (kind == 1) { if (c < M) idx = p.leaf_idx[(size_t)j * M + c]; }
+        else { if (c < p.prefix) idx = c; }
+        return (idx >= 0 && idx < p.nk) ? (int)idx : -1;
+    };
+    constexpr int kLoads = (kTileN * D / kVec + kThreads - 1) / kThreads;   // 16-byte pieces of K (and of V) per thread
+    float kreg[kLoads][kVec], vreg[kLoads][kVec];
+    auto fetch_rows = [&](const int* keys) {     // K/V rows of the tile whose key list is `keys` -> registers
+#pragma unroll
+        for (int it = 0; it < kLoads; ++it) {
+            const int e = tid + it * kThreads;
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) { kreg[it][i] = 0.f; vreg[it][i] = 0.f; }
+            if (e < kTileN * D / kVec) {
+                const int n = e / (D / kVec), d = (e % (D / kVec)) * kVec;
+                const int key = keys[n];
+                if (key >= 0) {
+                    load16(kb + (size_t)key * D + d, kreg[it]);
+                    load16(vb + (size_t)key * D + d, vreg[it]);
+                }
+            }
+        }
+    };
+    if (tid < kTileN) {
+        key_s[tid] = load_key(0);
+        key_s[kTileN + tid] = load_key(1);
+    }
+    __syncthreads();
+    if (total_tiles > 0) fetch_rows(key_s);
+
     for (int t = 0; t < total_tiles; ++t) {
-        // kind 0: ancestors, 1: leaves (diagonal), 2: shared prefix
-        int kind, base;
-        if (t < anc_tiles) { kind = 0; base = t * kTileN; }
-        else if (t < anc_tiles + leaf_tiles) { kind = 1; base = (t - anc_tiles) * kTileN; }
-        else { kind = 2; base = (t - anc_tiles - leaf_tiles) * kTileN; }
-
-        if (tid < kTileN) {
-            int64_t idx = -1;
-            const int c = base + tid;
-            if (kind == 0) { if (c < n_anc) idx = p.ancestor_idx[(size_t)j * p.max_anc + c]; }
-            else if (kind == 1) { if (c < M) idx = p.leaf_idx[(size_t)j * M + c]; }
-            else { if (c < p.prefix) idx = c; }
-            key_s[tid] = (idx >= 0 && idx < p.nk) ? (int)idx : -1;
-        }
-        __syncthreads();
-
-        for (int e = tid; e < kTileN * D / kVec; e += kThreads) {
-            const int n = e / (D / kVec), d = (e % (D / kVec)) * kVec;
-            const int key = key_s[n];
-            float kf[kVec], vf[kVec];
+        int base;
+        const int kind = tile_kind(t, base);
+        const int* keys = key_s + (t & 1) * kTileN;
+        // rows of tile t: registers -> LDS; then the requests for tile t + 1 and the list of tile t + 2
 #pragma unroll
-            for (int i = 0; i < kVec; ++i) { kf[i] = 0.f; vf[i] = 0.f; }
-            if (key >= 0) {
-                load16(kb + (size_t)key * D + d, kf);
-                load16(vb + (size_t)key * D + d, vf);
-            }
+        for (int it = 0; it < kLoads; ++it) {
+            const int e = tid + it * kThreads;
+            if (e < kTileN * D / kVec) {
+                const int n = e / (D / kVec), d = (e % (D / kVec)) * kVec;
 #pragma unroll
-            for (int i = 0; i < kVec; ++i) {
-                k_s[n * kPitch + d + i] = kf[i];
-                v_s[n * kPitch + d + i] = vf[i];
+                for (int i = 0; i < kVec; ++i) {
+                    k_s[n * kPitch + d + i] = kreg[it][i];
+                    v_s[n * kPitch + d + i] = vreg[it][i];
+                }
             }
         }
+        if (t + 1 < total_tiles) fetch_rows(key_s + ((t + 1) & 1) * kTileN);
+        int key_after_next = -1;
+        if (tid < kTileN) key_after_next = load_key(t + 2);
         __syncthreads();
 
         // scores of this thread's tile: rows sr + 32 i, keys sc .. sc + 3
@@ -160,7 +193,7 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     const int n = sc + c;
-                    bool ok = key_s[n] >= 0 && ((w >> n) & 1u);
+                    bool ok = keys[n] >= 0 && ((w >> n) & 1u);
                     if (kind == 1) ok = ok && (m == base + n);
                     s_s[m * kPitchS + n] = ok ? dot[i][c] * p.scale_log2e : -INFINITY;
                 }
@@ -212,6 +245,7 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
                 }
             }
         }
+        if (tid < kTileN) key_s[(t & 1) * kTileN + tid] = key_after_next;   // (tile t's list was last read in the score phase)
         __syncthreads();
     }
 
