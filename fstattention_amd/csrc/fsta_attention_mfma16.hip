@@ -92,6 +92,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     constexpr int kDmaWaves = kDmaPerTile < kWaves ? kDmaPerTile : kWaves;   // waves that gather
     constexpr int kDmaPerWave = kDmaPerTile / kDmaWaves;
     static_assert(kDmaPerWave * kDmaWaves == kDmaPerTile, "transfers must split evenly over the waves");
+    static_assert(kDmaPerWave == 1 || kDmaPerWave % 2 == 0, "a wave's transfers are K/V pairs of whole row groups");
     constexpr int kRowGroups = (kDmaPerWave + 1) / 2;   // row groups a wave touches per tile
     constexpr int kSteps = D / 32;                // MFMAs per 16-key half of S^T
     constexpr int kDTiles = D / 16;               // 16-row tiles of O^T
@@ -229,18 +230,29 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     // Lane i lands at LDS byte 16*i of the transfer, i.e. row i / kCpr, chunk slot i % kCpr, and
     // fetches the chunk that the XOR swizzle assigns to that slot.  Every gathering wave issues
     // exactly kDmaPerWave transfers per tile: the vmcnt bookkeeping counts on it.
+    // A lane's address is slice base (uniform) + a 32-bit byte offset: row * row pitch + the chunk
+    // its slot holds.  The chunk offsets are fixed for the kernel's life (dma_anc / dma_leaf); a
+    // request then costs one multiply-add per transfer.  (The launcher keeps slices below 4 GiB.)
+    uint32_t dma_anc[kDmaPerWave], dma_leaf[kDmaPerWave];
+#pragma unroll
+    for (int i = 0; i < kDmaPerWave; ++i) {
+        const int t2 = wave * kDmaPerWave + i;
+        const int r = (t2 >> 1) * kRowsPerDma + dma_row;
+        // V of a leaf tile is read row-wise like K (no transposing read), so it takes K's swizzle
+        dma_leaf[i] = (uint32_t)k_chunk<D>(r, dma_slot) * 16u;
+        dma_anc[i] = (t2 & 1) ? (uint32_t)v16_chunk<D>(r, dma_slot) * 16u : dma_leaf[i];
+    }
     auto issue_rows = [&](int t, int slot, const int (&rows)[kRowGroups]) {
         T* dst_tile = ring + slot * 2 * kTileElems;
+        const bool leaf_tile = t < kLeafTiles;
 #pragma unroll
         for (int i = 0; i < kDmaPerWave; ++i) {
             const int t2 = wave * kDmaPerWave + i;
             const int u = t2 >> 1;
             const bool is_v = t2 & 1;
-            const int r = u * kRowsPerDma + dma_row;
-            const size_t row_off = (size_t)rows[u - (wave * kDmaPerWave) / 2] * D;
-            // V of a leaf tile is read row-wise like K (no transposing read), so it takes K's swizzle
-            const T* src = is_v ? vb + row_off + (t < kLeafTiles ? k_chunk<D>(r, dma_slot) : v16_chunk<D>(r, dma_slot)) * 8
-                                : kb + row_off + k_chunk<D>(r, dma_slot) * 8;
+            const uint32_t off = (uint32_t)rows[i >> 1] * (uint32_t)(D * sizeof(T)) +
+                                 (leaf_tile ? dma_leaf[i] : dma_anc[i]);
+            const char* src = reinterpret_cast<const char*>(is_v ? vb : kb) + (size_t)off;
             __builtin_amdgcn_global_load_lds(
                 (const void __attribute__((address_space(1)))*)src,
                 (void __attribute__((address_space(3)))*)(dst_tile + (is_v ? kTileElems : 0) + u * 512),
@@ -345,11 +357,14 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     auto issue = [&](int t, int slot) {
         if (kDmaWaves < kWaves && wave >= kDmaWaves) return;
         int rows[kRowGroups];
+        if (kDShare || t < listed_tiles) {   // (head-dimension pairing is launched without a prefix)
 #pragma unroll
-        for (int i = 0; i < kRowGroups; ++i) {
-            const int r = ((wave * kDmaPerWave) / 2 + i) * kRowsPerDma + dma_row;
-            if (t < listed_tiles) rows[i] = key_s[t * kTileN + r];
-            else rows[i] = min((t + prefix_shift) * kTileN + r, p.prefix - 1);
+            for (int i = 0; i < kRowGroups; ++i)
+                rows[i] = key_s[t * kTileN + ((wave * kDmaPerWave) / 2 + i) * kRowsPerDma + dma_row];
+        } else {
+#pragma unroll
+            for (int i = 0; i < kRowGroups; ++i)
+                rows[i] = min((t + prefix_shift) * kTileN + ((wave * kDmaPerWave) / 2 + i) * kRowsPerDma + dma_row, p.prefix - 1);
         }
         issue_rows(t, slot, rows);
     };
@@ -824,6 +839,8 @@ int launch_d(const AttnParams& p, int head_dim, hipStream_t stream) {
 }  // namespace
 
 int launch_attention_mfma16(const AttnParams& p, int dtype, int head_dim, bool fast_pv, hipStream_t stream) {
+    // the gathers address a (batch, head) slice of K or V with 32-bit byte offsets
+    if ((uint64_t)p.nk * (uint64_t)head_dim * 2u > 0xffffffffull) return FSTA_EUNSUPPORTED;
     if (dtype == FSTA_F16) return launch_d<false, false>(p, head_dim, stream);
     if (fast_pv) return launch_d<true, false>(p, head_dim, stream);
     return launch_d<true, true>(p, head_dim, stream);
