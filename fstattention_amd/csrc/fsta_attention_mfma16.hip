@@ -119,24 +119,36 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
                  "s"(early_leaf), "s"(sub_shift));
 
     // Workgroup -> (slice, block), XCD-aware: every XCD gets whole (batch, head) slices, so all
-    // query blocks of a slice share one L2 for the K/V rows they have in common.
-    const int xcd = blockIdx.x % kXcds;
-    int within = blockIdx.x / kXcds;
-    // Key splits (long shared prefix, few blocks): workgroup `ksp` of a block takes the ksp-th run
+    // query blocks of a slice share one L2 for the K/V rows they have in common.  The grid is
+    // (8 XCDs x key runs, blocks, slices per XCD): workgroups go to the XCDs round-robin in x-fastest
+    // order and the x extent is a multiple of 8, so blockIdx.x % 8 is the XCD, and the blocks of
+    // a slice are dispatched next to each other.  (Grids past the y/z limits come as one long x
+    // axis in the same order: `linear_grid`.)
+    // Key runs (long shared prefix, few blocks): workgroup `ksp` of a block takes the ksp-th run
     // of prefix tiles, workgroup 0 also the tree part; each writes a normalised partial result
     // and its log-sum-exp, which a merge kernel joins.
-    int ksp = 0;
-    if constexpr (RUNS) {
-        ksp = within % p.key_splits;
-        within /= p.key_splits;
-    }
-    const bool tree = !RUNS || ksp == 0;
     // A workgroup takes M consecutive rows: a whole block of the caller's, or (sub_shift = 1, small
     // grids) one half of a block of 2M rows, so that twice as many CUs share the launch.  The
     // half-block reads the block's ancestor list and its own rows of the mask and leaf list.
-    const int parts = p.nb << sub_shift;
-    const int hz = (within / parts) * kXcds + xcd;
-    const int part = within % parts;
+    const int linear_grid = sub_shift >> 8;
+    sub_shift &= 0xff;
+    const int xcd = blockIdx.x % kXcds;
+    int ksp = 0, hz, part;
+    if (linear_grid) {
+        int within = blockIdx.x / kXcds;
+        if constexpr (RUNS) {
+            ksp = within % p.key_splits;
+            within /= p.key_splits;
+        }
+        const int parts = p.nb << sub_shift;
+        hz = (within / parts) * kXcds + xcd;
+        part = within % parts;
+    } else {
+        if constexpr (RUNS) ksp = blockIdx.x / kXcds;
+        hz = blockIdx.z * kXcds + xcd;
+        part = blockIdx.y;
+    }
+    const bool tree = !RUNS || ksp == 0;
     const int j = part >> sub_shift;                                        // block of the caller's lists
     const int block_rows = M << sub_shift;                                  // rows per such block
     const int row_base = j * block_rows + (part & ((1 << sub_shift) - 1)) * M;   // first query row of this workgroup
@@ -196,10 +208,10 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
                           ((size_t)j * p.mask_words * block_rows + (row_base - j * block_rows)) * 4;
         for (int piece = wave; piece * 64 < chunks; piece += kWaves) {
             const int c = piece * 64 + lane;
-            if (c < chunks)
+            if (c < chunks)   // (uniform base + 32-bit lane offset: a block's mask words are a few KiB)
                 __builtin_amdgcn_global_load_lds(
-                    (const void __attribute__((address_space(1)))*)(src + ((size_t)(c / (M / 4)) * block_rows * 4 +
-                                                                           (c % (M / 4)) * 16)),
+                    (const void __attribute__((address_space(1)))*)(src + (size_t)(uint32_t)((c / (M / 4)) * block_rows * 4 +
+                                                                                             (c % (M / 4)) * 16)),
                     (void __attribute__((address_space(3)))*)(reinterpret_cast<char*>(mask_s) + piece * 1024),
                     16, 0, 0);
         }
@@ -219,8 +231,9 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     for (int i = 0; i < kQDma; ++i) {
         const int r = i * kRowsPerDma + dma_row;
         const int grow = min(row_base + qgroup * 16 + r, p.nq - 1);
+        const uint32_t off = (uint32_t)grow * (uint32_t)(D * sizeof(T)) + (uint32_t)k_chunk<D>(r, dma_slot) * 16u;
         __builtin_amdgcn_global_load_lds(
-            (const void __attribute__((address_space(1)))*)(qb + (size_t)grow * D + k_chunk<D>(r, dma_slot) * 8),
+            (const void __attribute__((address_space(1)))*)(reinterpret_cast<const char*>(qb) + (size_t)off),
             (void __attribute__((address_space(3)))*)(qstage + i * 512), 16, 0, 0);
     }
 
@@ -763,7 +776,12 @@ int launch_ks(const AttnParams& p, int sub_shift, hipStream_t stream) {
     if (lds > 160 * 1024)
         return fail(FSTA_EUNSUPPORTED, "max_ancestors=%d needs %zu bytes of LDS (limit 163840)", p.max_anc, lds);
     const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
-    const unsigned grid = (unsigned)(kXcds * slices_per_xcd * (p.nb << sub_shift) * p.key_splits);
+    const unsigned grid = (unsigned)(kXcds * slices_per_xcd * (p.nb << sub_shift) * p.key_splits);   // workgroups
+    // (8 XCDs x key runs, blocks, slices per XCD) where the y and z extents allow it, else one axis
+    const bool linear_grid = (p.nb << sub_shift) > 65535 || slices_per_xcd > 65535;
+    const dim3 grid3 = linear_grid ? dim3(grid)
+                                   : dim3((unsigned)(kXcds * p.key_splits), (unsigned)(p.nb << sub_shift), (unsigned)slices_per_xcd);
+    const int shift_arg = sub_shift | (linear_grid ? 0x100 : 0);
     // a launch whose workgroups all run at once: leaf tiles requested early, Q in an area of its own
     constexpr size_t kQBytes = (size_t)kWaves * 16 * D * 2;
     const int early = grid <= kCus && p.key_splits == 1 && lds + kQBytes <= 160 * 1024 ? 1 : 0;
@@ -774,8 +792,8 @@ int launch_ks(const AttnParams& p, int sub_shift, hipStream_t stream) {
                 const int rc = allow_full_lds<&attn_mfma16_kernel<BF16, D, M, SPLIT, KS, true>>();
                 if (rc != FSTA_OK) return rc;
             }
-            hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT, KS, true>), dim3(grid), dim3(M * 4 * kShares),
-                               lds, stream, p, stages, early, sub_shift);
+            hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT, KS, true>), grid3, dim3(M * 4 * kShares),
+                               lds, stream, p, stages, early, shift_arg);
         } else {
             return FSTA_EUNSUPPORTED;   // (key runs are never combined with head-dimension shares)
         }
@@ -784,8 +802,8 @@ int launch_ks(const AttnParams& p, int sub_shift, hipStream_t stream) {
             const int rc = allow_full_lds<&attn_mfma16_kernel<BF16, D, M, SPLIT, KS, false>>();
             if (rc != FSTA_OK) return rc;
         }
-        hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT, KS, false>), dim3(grid), dim3(M * 4 * kShares), lds,
-                           stream, p, stages, early, sub_shift);
+        hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, SPLIT, KS, false>), grid3, dim3(M * 4 * kShares), lds,
+                           stream, p, stages, early, shift_arg);
     }
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
