@@ -141,6 +141,34 @@ def test_large_tree_behind_a_long_prefix_sampled_rows():
         sampled_rows_check(q, k, v, parent, o, lse, scale, prefix, 48, 66, torch.float16, f"large tree splits={splits}")
 
 
+def test_more_blocks_than_a_grid_axis_holds_sampled_rows():
+    """65538 blocks of 32 rows: past the 65535 limit of a grid's y axis, so the kernel is launched on
+    one long x axis and recovers (slice, block) by division.  The tree is a forest of 32-node trees,
+    one per block, whose kernel inputs are the first block's shifted.  Checked on sampled rows, and
+    every row against the vector-ALU kernel (independent code)."""
+    m, d, nb = 32, 32, 65538
+    one = trees.random_recursive_parents(m, 31, window=20)
+    lineage, level = trees.lineage_from_parents(one)
+    max_anc = trees.required_max_ancestors(one, m, 16)
+    a1, mask1, l1 = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), m, max_anc)
+    shift = torch.arange(nb, device="cuda", dtype=torch.int64)[:, None] * m
+    a_idx = torch.where(a1 >= 0, a1 + shift, a1).contiguous()
+    l_idx = torch.where(l1 >= 0, l1 + shift, l1).contiguous()
+    a_mask = mask1.expand(nb, m, max_anc).contiguous()
+    parent = np.tile(one, nb)
+    parent = np.where(parent >= 0, parent + np.repeat(np.arange(nb, dtype=np.int64) * m, m), -1)
+    nq = nb * m
+    g = torch.Generator(device="cuda").manual_seed(8)
+    q, k, v = (torch.randn((1, 1, nq, d), generator=g, device="cuda", dtype=torch.float16) for _ in range(3))
+    scale = 1.0 / math.sqrt(d)
+    o, lse = fst_attention(q, k, v, a_idx, a_mask, l_idx, scale, BLOCK_M=m, MAX_ANCESTORS=max_anc,
+                           out_dtype=torch.float32, return_lse=True)
+    sampled_rows_check(q, k, v, parent, o, lse, scale, 0, 64, 88, torch.float16, "65538 blocks")
+    other = fst_attention(q, k, v, a_idx, a_mask, l_idx, scale, BLOCK_M=m, MAX_ANCESTORS=max_anc,
+                          out_dtype=torch.float32, generic=True)
+    torch.testing.assert_close(o, other, atol=2e-3, rtol=2e-3)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("d", [16, 32, 64, 128])
 @pytest.mark.parametrize("block_m", [16, 32, 64, 128])
