@@ -299,13 +299,14 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         for (int i = 0; i < kKeyBatch; ++i) {
             const int c = c0 + i * kThreads;
             if (c < cap * kTileN) {
-                const bool ok = ids[i] >= 0 && ids[i] < p.nk;
+                const bool ok = (uint64_t)ids[i] < (uint64_t)p.nk;   // 0 <= id < nk
                 const uint64_t vote = __ballot(ok);
                 const uint32_t lo = (uint32_t)vote, hi = (uint32_t)(vote >> 32);   // two tiles per wave
                 const int mine_id = ok ? (int)ids[i] : 0;
-                // first valid row of each tile: wave-uniform lane numbers, so plain lane reads
-                const int first_lo = lo ? __builtin_amdgcn_readlane(mine_id, __ffs(lo) - 1) : 0;
-                const int first_hi = hi ? __builtin_amdgcn_readlane(mine_id, 31 + __ffs(hi)) : 0;
+                // first valid row of each tile: wave-uniform lane numbers, so plain lane reads.  A
+                // tile without a valid slot reads its last lane, which then holds row 0.
+                const int first_lo = __builtin_amdgcn_readlane(mine_id, __builtin_ctz(lo | 0x80000000u));
+                const int first_hi = __builtin_amdgcn_readlane(mine_id, 32 + __builtin_ctz(hi | 0x80000000u));
                 const uint32_t mine = lane < 32 ? lo : hi;
                 const int fallback = lane < 32 ? first_lo : first_hi;
                 lds_write_b32(lds_addr(key_s + c), ok ? (int)ids[i] : fallback);
