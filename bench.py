@@ -39,9 +39,9 @@ INFINITY_CACHE_BYTES = 256 << 20
 
 # HBM bytes per launch of the headline kernel (256-node tree, cold buffers) from two
 # rocprofv3 --pmc runs, see profiles/attn_mfma16_kernel_cfg2_medusa256_hbm_traffic.txt:
-# FETCH_SIZE 3174.5 KiB x 2.0 (a plain 256 MiB copy reads 131084 KiB on this counter, i.e. the
+# FETCH_SIZE 3155.5 KiB x 2.0 (a plain 256 MiB copy reads 131084 KiB on this counter, i.e. the
 # counter sees half of the read traffic) + WRITE_SIZE 2080 KiB x 1.0 (the copy reads 262144).
-MEASURED_TRAFFIC_BYTES = int((3174.5 * 2 + 2080) * 1024)
+MEASURED_TRAFFIC_BYTES = int((3155.5 * 2 + 2080) * 1024)
 
 
 def parse_args():
