@@ -124,6 +124,9 @@ int fsta_pack_mask(const int64_t* ancestor_idx, const uint8_t* ancestor_mask,
  * gets o = 0 and lse = -inf.
  * head_dim in {16,32,64,128}; block_m in {16,32,64,128}; max_ancestors >= 1.
  * q, k, v and o must be 16-byte aligned (rows are moved 16 bytes at a time).
+ * batch * heads <= 65535.  The matrix-core kernels address one (batch, head)
+ * slice of K or V with 32-bit byte offsets: slices of 4 GiB and more
+ * (nk * head_dim * 2 bytes) are served by the slower vector-ALU kernel.
  */
 int fsta_attention_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                        const int64_t* ancestor_idx, const uint32_t* mask_bits,
