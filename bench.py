@@ -59,6 +59,9 @@ def parse_args():
                          "(reference point for the FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--dtype", choices=["bf16", "f16", "f32"], default=None,
                     help="storage type of q/k/v (default: the configuration's own, bf16 for the headline)")
+    ap.add_argument("--prefix", type=int, default=0, metavar="KEYS",
+                    help="put a shared dense prefix of KEYS keys in front of the tree (reference "
+                         "fstattention.py:113-136); not the headline workload, implies --no-cpu")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-graph", action="store_true", help="time plain stream launches only")
     return ap.parse_args()
@@ -454,7 +457,7 @@ def main():
     use_graph = not args.no_graph
 
     dtype = {None: None, "bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[args.dtype]
-    wl = Workload(args.config, sets_bytes=2 * INFINITY_CACHE_BYTES, dtype=dtype)
+    wl = Workload(args.config, sets_bytes=2 * INFINITY_CACHE_BYTES, dtype=dtype, prefix=args.prefix)
     ok, max_err, tol = wl.cross_check()
     if not ok:
         print(f"bench.py: the two kernels disagree (max difference {max_err:.3e} > {tol})", file=sys.stderr)
@@ -466,7 +469,8 @@ def main():
     achieved = wl.kv_bytes / kernel_s / 1e9
     result = {
         "metric": "K/V GB/s loaded (us/call in us_per_call), 256-node Medusa tree H32 D128 bf16"
-                  if args.config == 2 else f"K/V GB/s loaded, {wl.cfg.name}",
+                  if args.config == 2 and not args.prefix else
+                  f"K/V GB/s loaded, {wl.cfg.name}" + (f" behind {args.prefix} prefix keys" if args.prefix else ""),
         "value": round(wl.kv_bytes / step_s / 1e9, 2),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -480,7 +484,7 @@ def main():
         "dtype": {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[wl.dtype],
         "data": "synthetic",
         "config": {
-            "workload": wl.cfg.name, "nodes": wl.n, "batch": wl.z, "heads": wl.h, "head_dim": wl.d,
+            "workload": wl.cfg.name + (f"_prefix{args.prefix}" if args.prefix else ""), "nodes": wl.n, "batch": wl.z, "heads": wl.h, "head_dim": wl.d,
             "block_m": wl.m, "max_ancestors": wl.max_anc, "kv_rows_per_head": wl.kv_rows,
             "kv_bytes_per_call": wl.kv_bytes, "attended_pairs": wl.pairs, "flops_per_call": wl.flops,
             "timed_region": ("hip graph of K steps" if use_graph else "K stream launches") +
@@ -492,12 +496,12 @@ def main():
             "bound": "hbm",
             "kernel": ("attn_generic_kernel" if wl.dtype == torch.float32 else
                        "attn_mfma16_kernel<bf16, D=128, 32-row halves of the 64-row blocks, split P, wave pairs by head-dim halves>"
-                       if args.config == 2 and wl.dtype == torch.bfloat16 else "attn_mfma16_kernel"),
+                       if args.config == 2 and wl.dtype == torch.bfloat16 and not args.prefix else "attn_mfma16_kernel"),
             "achieved": round(achieved, 2),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 5),
-            "traffic": MEASURED_TRAFFIC_BYTES if args.config == 2 else None,
+            "traffic": MEASURED_TRAFFIC_BYTES if args.config == 2 and not args.prefix else None,
             "algorithmic_bytes_per_launch": wl.kv_bytes,
             "avg_launch_us": round(kernel_s * 1e6, 3),
             "mfma_frac_of_bf16_peak": round(wl.flops / kernel_s / 1e12 / MFMA_BF16_PEAK_TFLOPS, 6),
@@ -510,7 +514,10 @@ def main():
             "python_api_warm": round(time_python_api(wl, args.steps, args.warmup) * 1e6, 3),
             "gpu_precompute": round(time_precompute(wl) * 1e6, 3),
         }
-    if not args.no_cpu:
+    if args.prefix:
+        result["config"]["prefix_keys"] = args.prefix
+        result["config"]["key_runs"] = int(wl.key_runs)
+    if not args.no_cpu and not args.prefix:
         result["cpu_baseline"], result["parity"] = cpu_baseline(wl)
         if not result["parity"]["ok"]:
             print(f"bench.py: parity against the CPU oracle failed: {result['parity']}", file=sys.stderr)
