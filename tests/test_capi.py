@@ -31,6 +31,35 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"{name} is declared in fsta.h but not exported"
 
 
+def test_header_is_plain_c_and_a_c_program_links(tmp_path):
+    """include/fsta.h is what a C, cgo or FFI binding includes: it has to compile as C99 without the
+    HIP headers, and a C program has to link against the library and reach its host-side checks."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.fail(f"{_lib.LIB_PATH} has not been built (python -m fstattention_amd.build)")
+    src = tmp_path / "use_fsta.c"
+    src.write_text(
+        '#include "fsta.h"\n#include <stdio.h>\n#include <string.h>\n'
+        "int main(void) {\n"
+        "    if (fsta_abi_version() != FSTA_ABI_VERSION) return 1;\n"
+        "    if (fsta_mask_words(80) != 3) return 2;\n"
+        "    /* rejected on the host, before any GPU work: head_dim 48 is not supported */\n"
+        "    int rc = fsta_attention_fwd(0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 1, 64, 64, 48, FSTA_BF16, FSTA_BF16,\n"
+        "                                64, 64, 1, 0.125f, 0, 0);\n"
+        "    if (rc == FSTA_OK || strlen(fsta_last_error()) == 0) return 3;\n"
+        '    printf("ok\\n");\n    return 0;\n}\n')
+    exe = tmp_path / "use_fsta"
+    libdir = os.path.dirname(_lib.LIB_PATH)
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.dirname(HEADER),
+                    str(src), "-o", str(exe), "-L", libdir, "-l:" + os.path.basename(_lib.LIB_PATH),
+                    "-Wl,-rpath," + libdir, "-Wl,--allow-shlib-undefined"], check=True, capture_output=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0 and out.stdout.strip() == "ok", (out.returncode, out.stdout, out.stderr)
+
+
 def test_constants_match_header():
     text = open(HEADER).read()
     defs = dict(re.findall(r"#define\s+(FSTA_[A-Z_0-9]+)\s+(-?\d+)u?\b", text))
