@@ -564,6 +564,43 @@ def test_hip_graph_replays_match_eager_calls():
     assert_close(out, want, cfg.dtype, "last replay")
 
 
+def test_hip_graph_replays_of_key_runs_match_eager_calls():
+    """A long shared prefix cut into runs of keys (two kernels and a workspace from torch's graph-private
+    pool) captured into a HIP graph; replays on new q and new prefix rows must give the eager results."""
+    cfg = trees.config(2)
+    m, d, prefix = cfg.block_m, cfg.head_dim, 3000
+    lineage, level = trees.lineage_from_parents(cfg.parent)
+    max_anc = trees.required_max_ancestors(cfg.parent, m)
+    a_idx, a_mask, l_idx = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), m, max_anc)
+    a_idx, l_idx = shift_for_prefix(a_idx, l_idx, prefix)
+    scale = 1.0 / math.sqrt(d)
+    q, k, v = (t.cuda() for t in rand_qkv(1, 2, cfg.n_nodes, prefix + cfg.n_nodes, d, cfg.dtype, 41))
+
+    def step():
+        return fst_attention(q, k, v, a_idx, a_mask, l_idx, scale, BLOCK_M=m, MAX_ANCESTORS=max_anc,
+                             out_dtype=torch.float32, key_splits=5)
+
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        step()
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            out = step()
+    for replay in range(3):
+        g = torch.Generator().manual_seed(200 + replay)
+        q.copy_(torch.randn(q.shape, generator=g).to(q.dtype))
+        k[:, :, :prefix].copy_(torch.randn((1, 2, prefix, d), generator=g).to(k.dtype))
+        eager = step().clone()
+        torch.cuda.synchronize()
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {replay} differs from the eager call"
+    want, _ = dense_oracle(q.cpu(), k.cpu(), v.cpu(), cfg.parent, scale, prefix=prefix)
+    assert_close(out, want, cfg.dtype, "last replay")
+
+
 def test_decoding_step_from_probabilities_in_one_graph():
     """Draft-head probabilities -> tree -> depth-first order -> lineage -> kernel inputs -> attention,
     captured once as one HIP graph; every replay reads new probabilities (a different tree) and new
