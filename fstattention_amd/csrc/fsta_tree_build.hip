@@ -11,8 +11,9 @@
 // of a path is the path without its last rank.
 //
 //   1. scores of all candidates into LDS
-//   2. the (n-1)-th largest score by radix selection on the bit patterns (8 passes of 8 bits;
-//      non-negative doubles order like their bit patterns)
+//   2. the (n-1)-th largest score by radix selection on the bit patterns (up to 8 passes of 8 bits,
+//      ending as soon as the candidates left all belong to the kept ones; non-negative doubles
+//      order like their bit patterns)
 //   3. "kept" flags (above the threshold, or equal to it and among the first ties), numbered by
 //      a prefix sum over the candidate index
 //   4. parent ids through the numbering of the parents' candidates
@@ -36,7 +37,7 @@ __global__ __launch_bounds__(kBuildThreads) void medusa_tree_kernel(const T* __r
     uint64_t* key_s = reinterpret_cast<uint64_t*>(build_s);                    // [n_cand] score bits, later node ids
     double* prob_s = reinterpret_cast<double*>(key_s + n_cand);                // [depths * topk]
     uint32_t* hist_s = reinterpret_cast<uint32_t*>(prob_s + depths * topk);    // [256] bytes; later counts per (row, wave)
-    uint32_t* misc_s = hist_s + 256;   // [0] chosen byte, [1] candidates still wanted
+    uint32_t* misc_s = hist_s + 256;   // [0] chosen byte, [1] candidates still wanted, [2] selection finished
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -47,7 +48,7 @@ __global__ __launch_bounds__(kBuildThreads) void medusa_tree_kernel(const T* __r
         return;
     }
     for (int e = tid; e < depths * topk; e += kBuildThreads) prob_s[e] = (double)probs[e];
-    if (tid < 2) misc_s[tid] = 0u;
+    if (tid < 3) misc_s[tid] = 0u;
     __syncthreads();
 
     // 1. scores, depth by depth: a path's score is its prefix's score times the probability of
@@ -126,6 +127,8 @@ __global__ __launch_bounds__(kBuildThreads) void medusa_tree_kernel(const T* __r
                 if (before < want && want <= before + mine[b]) {
                     misc_s[0] = (uint32_t)(255 - 4 * tid - b);
                     misc_s[1] = want - before;
+                    // every candidate of this byte value is wanted: the lower bytes need no look
+                    if (want - before == mine[b]) misc_s[2] = 1u;
                 }
                 before += mine[b];
             }
@@ -133,6 +136,8 @@ __global__ __launch_bounds__(kBuildThreads) void medusa_tree_kernel(const T* __r
         __syncthreads();
         prefix |= (uint64_t)misc_s[0] << shift;
         want = misc_s[1];
+        // (uniform: everyone reads the flag between the same two barriers)
+        if (misc_s[2] != 0u) break;   // threshold = the prefix with zero lower bytes, all `want` candidates from it up
     }
     // prefix = the threshold; `want` of the candidates equal to it are kept, the first ones by index
     const uint64_t threshold = prefix;
