@@ -304,9 +304,9 @@ def time_front_end(index, reps=20, stages=None):
     return {name: device_us(fn) for name, fn in calls.items() if stages is None or name in stages}
 
 
-def time_decoding_step(wl, layers=32, reps=5):
+def time_decoding_step(wl, layers=32, reps=5, depth_first=True):
     """One decoding step of the headline workload as one HIP graph: draft probabilities -> tree ->
-    depth-first order -> lineage -> kernel inputs (once), then `layers` attention calls on rotating
+    (depth-first order ->) lineage -> kernel inputs (once), then `layers` attention calls on rotating
     q/k/v/o sets that all use those inputs.  Microseconds per step from HIP events."""
     import torch
     from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, fst_attention,
@@ -318,9 +318,10 @@ def time_decoding_step(wl, layers=32, reps=5):
     def step():
         status = torch.zeros((1,), dtype=torch.int32, device=dev)
         parent = medusa_parents_gpu(probs, wl.n, status=status)
-        perm, rank = dfs_order_gpu(parent, "light_first", check=False, status=status)
-        new_parent = renumber_parents_gpu(parent, perm, rank)
-        lineage, level = lineage_from_parents_gpu(new_parent, width=depths + 1, check=False, status=status)
+        if depth_first:
+            perm, rank = dfs_order_gpu(parent, "light_first", check=False, status=status)
+            parent = renumber_parents_gpu(parent, perm, rank)
+        lineage, level = lineage_from_parents_gpu(parent, width=depths + 1, check=False, status=status)
         a_idx, packed, l_idx, _ = create_fst_attention_kernel_inputs(
             lineage, level, wl.m, wl.max_anc, check=False, want_bool_mask=False, status=status)
         for layer in range(layers):
@@ -575,11 +576,13 @@ def main():
             }
             del w
             torch.cuda.empty_cache()
-        step_us = time_decoding_step(wl)
         extra["cfg2_decoding_step"] = {
-            "layers": 32, "total_us": round(step_us, 1),
-            "note": "one graph: probabilities -> tree -> depth-first order -> lineage -> kernel inputs, then 32 "
-                    "attention calls (Python wrapper, output allocated per call) on rotating q/k/v sets",
+            "layers": 32,
+            "total_us": round(time_decoding_step(wl, depth_first=False), 1),
+            "total_us_depth_first_order": round(time_decoding_step(wl), 1),
+            "note": "one graph: probabilities -> tree (-> depth-first order) -> lineage -> kernel inputs, then 32 "
+                    "attention calls (Python wrapper, output allocated per call) on rotating q/k/v sets; a tree "
+                    "this small gains nothing from the depth-first order, the large ones do",
         }
         # the integer kernels that turn a new tree into kernel inputs once per decoding step
         extra["front_end_device_us"] = {trees_name: time_front_end(idx) for idx, trees_name in
