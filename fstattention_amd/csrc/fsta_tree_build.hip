@@ -147,8 +147,9 @@ __global__ __launch_bounds__(kBuildThreads) void medusa_tree_kernel(const T* __r
     //    an exclusive scan over those 256 counts, and the lanes below within the wave.
     uint32_t* count_s = hist_s;
     __syncthreads();
+    if (tid < 256 && tid >= rows * kBuildWaves) count_s[tid] = 0u;   // rows this launch does not have
 #pragma unroll 1
-    for (int k = 0; k < kBuildRows; ++k) {
+    for (int k = 0; k < rows; ++k) {
         const int c = tid + k * kBuildThreads;
         const uint64_t key = c < n_cand ? key_s[c] : 0ull;
         const uint64_t over = __ballot(c < n_cand && key > threshold);
