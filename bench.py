@@ -106,7 +106,8 @@ class Workload:
         self.nk = self.n + prefix
         if prefix:
             self.a_idx, self.l_idx = shift_for_prefix(self.a_idx, self.l_idx, prefix)
-        self.packed = _packed_for(self.a_idx, self.a_mask)
+        self.packed = _packed_for(self.a_idx, self.a_mask, self.l_idx, self.nk)
+        self.plan_ptr = self.packed.plan.data_ptr() if self.packed.plan is not None else None
         self.nb = self.a_idx.shape[0]
         rows = int((self.a_idx >= 0).sum().item() + (self.l_idx >= 0).sum().item())
         self.kv_rows = rows + self.nb * prefix       # every block walks the whole prefix
@@ -154,14 +155,16 @@ class Workload:
             self._check(self.lib.fsta_attention_fwd_ws(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), self.lse.data_ptr(),
                 self.a_idx.data_ptr(), self.packed.mask_bits.data_ptr(), self.packed.anc_count.data_ptr(),
-                self.l_idx.data_ptr(), self.z, self.h, self.n, self.nk, self.d, self.code, self.code,
+                self.l_idx.data_ptr(), self.plan_ptr, self.packed.key_shift,
+                self.z, self.h, self.n, self.nk, self.d, self.code, self.code,
                 self.m, self.max_anc, self.nb, self.scale, flags | self.flags, self.work.data_ptr(),
                 self.work.numel(), torch.cuda.current_stream().cuda_stream))
             return
         self._check(self.lib.fsta_attention_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), self.lse.data_ptr(),
             self.a_idx.data_ptr(), self.packed.mask_bits.data_ptr(), self.packed.anc_count.data_ptr(),
-            self.l_idx.data_ptr(), self.z, self.h, self.n, self.nk, self.d, self.code, self.code,
+            self.l_idx.data_ptr(), self.plan_ptr, self.packed.key_shift,
+            self.z, self.h, self.n, self.nk, self.d, self.code, self.code,
             self.m, self.max_anc, self.nb, self.scale, flags | self.flags,
             torch.cuda.current_stream().cuda_stream))
 

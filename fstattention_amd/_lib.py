@@ -19,25 +19,26 @@ def flag_key_splits(n: int) -> int:
 
 PRE_TOO_MANY_ANCESTORS, PRE_BAD_NODE_ID, PRE_BAD_LEVEL = 1, 2, 4
 TREE_NOT_PREFIX_CLOSED = 8
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 # name -> (restype, argtypes); every symbol include/fsta.h declares
 SIGNATURES = {
     "fsta_abi_version": (c_int, []),
     "fsta_last_error": (c_char_p, []),
     "fsta_mask_words": (c_int32, [c_int32]),
+    "fsta_block_plan_bytes": (c_size_t, [c_int32, c_int32, c_int32]),
     "fsta_precompute": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int32, c_int32,
-                                c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
-    "fsta_pack_mask": (c_int, [c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p, c_void_p,
-                               c_void_p]),
+                                c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "fsta_pack_mask": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int64, c_void_p, c_void_p,
+                               c_void_p, c_void_p]),
     "fsta_attention_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                   c_void_p, c_void_p, c_void_p, c_void_p,
+                                   c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32,
                                    c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
                                    c_int32, c_int32, c_int32, c_float, c_uint32, c_void_p]),
     "fsta_attention_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
                                                   c_int32, c_float, c_uint32]),
     "fsta_attention_fwd_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                      c_void_p, c_void_p, c_void_p, c_void_p,
+                                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32,
                                       c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
                                       c_int32, c_int32, c_int32, c_float, c_uint32, c_void_p, c_size_t, c_void_p]),
     "fsta_lineage_from_parents": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p,

@@ -16,15 +16,25 @@ _DTYPES = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _li
 
 
 class PackedTreeMask(NamedTuple):
-    """Bit-packed form of ``ancestor_mask`` the kernels read.
+    """Kernel-ready form of the per-block inputs.
 
     ``mask_bits`` uint32-as-int32 ``[NB, ceil(A/32), M]`` (bit ``b`` of word ``w``
     of row ``r`` = ``ancestor_mask[j, r, 32*w + b]``), ``anc_count`` int32 ``[NB]``.
+    ``plan`` (int32, or ``None`` for block sizes other than 32/64/128): the block plan of
+    ``include/fsta.h`` -- 32-bit K/V rows of every ancestor and leaf slot, leaf validity and the
+    mask words, per block, in the order the matrix-core kernel consumes them; it belongs to the
+    ``ancestor_idx`` / ``leaf_idx`` it was made from.  ``key_shift``: what has been added to the
+    valid entries of those tensors since (``shift_for_prefix``); the kernel adds it to the plan's
+    keys.  ``key_limit``: ids at or above it were treated as empty slots when the plan was made
+    (``None``: the plan comes from the tree precompute and holds tree nodes only).
     """
     mask_bits: torch.Tensor
     anc_count: torch.Tensor
     block_m: int
     max_ancestors: int
+    plan: Optional[torch.Tensor] = None
+    key_shift: int = 0
+    key_limit: Optional[int] = None
 
 
 def _stream_ptr(device) -> int:
@@ -55,8 +65,11 @@ class _on_device:
         return False
 
 
-def pack_tree_mask(ancestor_idx: torch.Tensor, ancestor_mask: torch.Tensor) -> PackedTreeMask:
-    """bool ``[NB, M, A]`` mask (+ ``ancestor_idx`` for the ``-1`` slots) -> packed bits."""
+def pack_tree_mask(ancestor_idx: torch.Tensor, ancestor_mask: torch.Tensor,
+                   leaf_idx: Optional[torch.Tensor] = None, key_limit: Optional[int] = None) -> PackedTreeMask:
+    """bool ``[NB, M, A]`` mask (+ ``ancestor_idx`` for the ``-1`` slots) -> packed bits; with
+    ``leaf_idx`` ``[NB, M]`` (and a block size of 32, 64 or 128) also the block plan, in which
+    ids outside ``[0, key_limit)`` count as empty slots (``key_limit``: rows of K/V)."""
     if not ancestor_mask.is_cuda or not ancestor_idx.is_cuda:
         raise ValueError("pack_tree_mask needs tensors on the GPU")
     if ancestor_mask.dtype != torch.bool or ancestor_idx.dtype != torch.int64:
@@ -73,32 +86,65 @@ def pack_tree_mask(ancestor_idx: torch.Tensor, ancestor_mask: torch.Tensor) -> P
     words = (a + 31) // 32
     bits = torch.empty((nb, words, m), dtype=torch.int32, device=dev)
     count = torch.empty((nb,), dtype=torch.int32, device=dev)
+    plan, limit = None, None
+    plan_bytes = lib.fsta_block_plan_bytes(nb, m, a) if leaf_idx is not None and a <= 16384 else 0
+    if plan_bytes:
+        if leaf_idx.dtype != torch.int64 or tuple(leaf_idx.shape) != (nb, m) or leaf_idx.device != dev:
+            raise ValueError(f"leaf_idx must be int64 [{nb}, {m}] on {dev}")
+        leaf_idx = leaf_idx.contiguous()
+        plan = torch.empty((plan_bytes // 4,), dtype=torch.int32, device=dev)
+        limit = _MAX_KEY if key_limit is None else min(int(key_limit), _MAX_KEY)
     with _on_device(dev):
-        _lib.check(lib.fsta_pack_mask(ancestor_idx.data_ptr(), ancestor_mask.data_ptr(), nb, m, a,
-                                      bits.data_ptr(), count.data_ptr(), _stream_ptr(dev)))
-    return PackedTreeMask(bits, count, m, a)
+        _lib.check(lib.fsta_pack_mask(ancestor_idx.data_ptr(), ancestor_mask.data_ptr(),
+                                      leaf_idx.data_ptr() if plan is not None else None, nb, m, a,
+                                      limit if plan is not None else 0, bits.data_ptr(), count.data_ptr(),
+                                      plan.data_ptr() if plan is not None else None, _stream_ptr(dev)))
+    return PackedTreeMask(bits, count, m, a, plan, 0, limit)
 
 
-def _packed_for(ancestor_idx: torch.Tensor, ancestor_mask) -> PackedTreeMask:
-    """Packed mask of a bool tensor, remembered on the tensor object.
+_MAX_KEY = 2 ** 31 - 1
+
+
+def _version(t: torch.Tensor):
+    """torch's in-place edit counter of `t`, or None for tensors that keep none (tensors made
+    under ``torch.inference_mode()``)."""
+    try:
+        return t._version
+    except RuntimeError:
+        return None
+
+
+def _cache_key(ancestor_idx, ancestor_mask, leaf_idx):
+    """What a packed copy kept on ``ancestor_mask`` was made from, or None when in-place edits of
+    one of the three tensors could not be noticed."""
+    versions = (_version(ancestor_mask), _version(ancestor_idx), _version(leaf_idx))
+    if None in versions:
+        return None
+    return versions + (ancestor_idx.data_ptr(), leaf_idx.data_ptr(), tuple(ancestor_mask.shape))
+
+
+def _packed_for(ancestor_idx: torch.Tensor, ancestor_mask, leaf_idx: torch.Tensor, nk: int) -> PackedTreeMask:
+    """Packed mask and block plan of a bool tensor, remembered on the tensor object.
 
     The kernel inputs are built once per decoding step and reused by every
     layer; the packed copy is kept as an attribute of ``ancestor_mask`` and
-    dropped when either tensor has been written to since (torch's version
-    counters) or ``ancestor_idx`` is a different tensor.
+    dropped when one of the three tensors has been written to since (torch's version
+    counters), ``ancestor_idx`` or ``leaf_idx`` is a different tensor, or K/V have another number
+    of rows than the plan was made for.  Tensors without version counters (inference mode) are
+    packed on every call; pass a :class:`PackedTreeMask` to avoid that.
     """
     if isinstance(ancestor_mask, PackedTreeMask):
         return ancestor_mask
-    key = (ancestor_mask._version, ancestor_idx.data_ptr(), ancestor_idx._version,
-           tuple(ancestor_mask.shape))
-    cached = getattr(ancestor_mask, "_fsta_packed", None)
-    if cached is not None and cached[0] == key:
+    key = _cache_key(ancestor_idx, ancestor_mask, leaf_idx)
+    cached = getattr(ancestor_mask, "_fsta_packed", None) if key is not None else None
+    if cached is not None and cached[0] == key and cached[1].key_limit in (None, nk):
         return cached[1]
-    packed = pack_tree_mask(ancestor_idx, ancestor_mask)
-    try:
-        ancestor_mask._fsta_packed = (key, packed)
-    except AttributeError:
-        pass
+    packed = pack_tree_mask(ancestor_idx, ancestor_mask, leaf_idx, nk)
+    if key is not None:
+        try:
+            ancestor_mask._fsta_packed = (key, packed)
+        except AttributeError:
+            pass
     return packed
 
 
@@ -171,7 +217,8 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
     lib = _lib.load()
     ancestor_idx = ancestor_idx.contiguous()
     leaf_idx = leaf_idx.contiguous()
-    packed = _packed_for(ancestor_idx, ancestor_mask)
+    packed = _packed_for(ancestor_idx, ancestor_mask, leaf_idx, Nk)
+    plan_ptr = packed.plan.data_ptr() if packed.plan is not None else None
     o = torch.empty(q.shape, dtype=out_dtype, device=q.device)
     # the reference allocates L and drops it (fstattention.py:158-160,181); here it only exists when asked for
     lse = torch.empty((Z * H, Nq), device=q.device, dtype=torch.float32) if return_lse else None
@@ -189,21 +236,28 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
         _lib.check(lib.fsta_attention_fwd_ws(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr() if return_lse else None,
             ancestor_idx.data_ptr(), packed.mask_bits.data_ptr(), packed.anc_count.data_ptr(),
-            leaf_idx.data_ptr(), Z, H, Nq, Nk, D, _DTYPES[q.dtype], _DTYPES[out_dtype],
+            leaf_idx.data_ptr(), plan_ptr, packed.key_shift, Z, H, Nq, Nk, D, _DTYPES[q.dtype], _DTYPES[out_dtype],
             BLOCK_M, MAX_ANCESTORS, nb, float(sm_scale), flags,
             work.data_ptr() if work is not None else None, work_bytes, _stream_ptr(q.device)))
     return (o, lse) if return_lse else o
 
 
-def shift_for_prefix(ancestor_idx: torch.Tensor, leaf_idx: torch.Tensor, prefix: int):
+def shift_for_prefix(ancestor_idx: torch.Tensor, leaf_idx: torch.Tensor, prefix: int,
+                     packed: Optional[PackedTreeMask] = None):
     """Index tensors for K/V laid out as ``[prefix | tree]``.
 
     The reference's caller adds the prefix length to every entry
     (``fstattention.py:211-212``), which turns the ``-1`` sentinels into the
-    valid row ``prefix-1``; this shifts real entries only.
+    valid row ``prefix-1``; this shifts real entries only.  With ``packed`` (the
+    :class:`PackedTreeMask` that belongs to the two tensors) a third value is returned: the same
+    packed inputs with the shift noted, so that they stay valid for the shifted tensors.
     """
-    return (torch.where(ancestor_idx >= 0, ancestor_idx + prefix, ancestor_idx),
-            torch.where(leaf_idx >= 0, leaf_idx + prefix, leaf_idx))
+    shifted = (torch.where(ancestor_idx >= 0, ancestor_idx + prefix, ancestor_idx),
+               torch.where(leaf_idx >= 0, leaf_idx + prefix, leaf_idx))
+    if packed is None:
+        return shifted
+    limit = None if packed.key_limit is None else packed.key_limit + prefix
+    return shifted + (packed._replace(key_shift=packed.key_shift + prefix, key_limit=limit),)
 
 
 def merge_attention_states(o_a: torch.Tensor, lse_a: torch.Tensor, o_b: torch.Tensor, lse_b: torch.Tensor):

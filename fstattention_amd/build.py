@@ -34,7 +34,12 @@ HIPCC_FLAGS = [
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option", "-Wno-option-ignored",
+    "-Rpass-analysis=kernel-resource-usage",
 ]
+
+# Kernels of these sources must keep everything in registers: a private array the compiler leaves
+# in scratch memory, or a spill, is reloaded through the same vmcnt queue their gather rings count on.
+NO_SCRATCH = ("fsta_attention_mfma16.hip", "fsta_attention_mfma.hip")
 
 
 def _hipcc() -> str:
@@ -51,6 +56,29 @@ def _run(cmd):
     return proc.stderr
 
 
+def _split_resource_remarks(stderr: str):
+    """hipcc's -Rpass-analysis=kernel-resource-usage remarks -> ({kernel: {field: int}}, the other lines)."""
+    usage, rest, current, skip = {}, [], None, 0
+    for line in stderr.splitlines():
+        if skip:                      # the two source-quote lines clang prints under the first remark of a kernel
+            skip -= 1
+            continue
+        if "[-Rpass-analysis=kernel-resource-usage]" in line:
+            body = line.split("remark:", 1)[1].rsplit("[-Rpass", 1)[0].strip()
+            key, _, val = body.rpartition(":")
+            if key.strip() == "Function Name":
+                current = usage.setdefault(val.strip(), {})
+                skip = 2
+            elif current is not None:
+                try:
+                    current[key.strip()] = int(val)
+                except ValueError:
+                    pass
+            continue
+        rest.append(line)
+    return usage, "\n".join(rest)
+
+
 def build_library(verbose: bool = True, jobs: int | None = None) -> str:
     """Compiles every source and links ``libfsta.so``; always rebuilds."""
     hipcc = _hipcc()
@@ -64,7 +92,13 @@ def build_library(verbose: bool = True, jobs: int | None = None) -> str:
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         results = list(pool.map(compile_one, SOURCES))
-    for _, warn in results:
+    for (obj, warn), src in zip(results, SOURCES):
+        usage, warn = _split_resource_remarks(warn)
+        if src in NO_SCRATCH:
+            bad = [(name, u) for name, u in usage.items() if u.get("ScratchSize [bytes/lane]", 0)]
+            if bad:
+                raise RuntimeError(f"{src}: kernels using scratch memory: " +
+                                   ", ".join(f"{n} ({u['ScratchSize [bytes/lane]']} B/lane)" for n, u in bad))
         # hipcc's host pass does not know the device-only feature name: not a problem
         warn = "\n".join(l for l in warn.splitlines() if "packed-fp32-ops" not in l)
         if verbose and warn.strip():

@@ -38,11 +38,12 @@ template <int D> __device__ __forceinline__ int v16_chunk(int row, int c) {
     return c ^ (2 * ((row / rpb) % gpr));
 }
 
+// LDS of one workgroup: the ring of K|V tiles, then the workgroup's part of the block plan
+// (header and ancestor keys, then leaf keys and mask words of its M/32 groups of 32 rows).
 template <int D, int M>
-__host__ __device__ constexpr size_t mfma16_lds_bytes(int max_anc, int stages) {
-    return (size_t)stages * 2 * kTileN * D * 2 +
-           (size_t)(M / 32 + anc_tile_capacity(max_anc)) * (kTileN * 4 + 4) + 12 + 32 +
-           (size_t)anc_tile_capacity(max_anc) * M * 4;
+__host__ __device__ inline size_t mfma16_lds_bytes(int max_anc, int stages) {
+    const PlanLayout l = plan_layout(M, max_anc);
+    return (size_t)stages * 2 * kTileN * D * 2 + (size_t)l.block_words * 4;
 }
 
 // 16 staged rows of W bytes each (LDS, `stride` apart) -> global rows `pitch` apart, 16 bytes per
@@ -85,7 +86,6 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     static_assert(!kDShare || (KS == -2 && D >= 64), "head-dimension halves need two accumulator tiles each");
     constexpr int kLeafGroup = leaf_group16_for(M);
     constexpr int kWaves = kQGroups * kShares;
-    constexpr int kThreads = kWaves * 64;
     constexpr int kCpr = D / 8;                   // 16-byte chunks per row
     constexpr int kRowsPerDma = 64 / kCpr;        // rows one wave-wide 1 KiB transfer covers
     constexpr int kDmaPerTile = 2 * kTileN / kRowsPerDma;   // K and V transfers of one tile
@@ -104,19 +104,19 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     T* ring = reinterpret_cast<T*>(smem);                 // [stages][K tile | V tile]
-    int* key_s = reinterpret_cast<int*>(ring + stages * 2 * kTileElems);
-    const int cap = kLeafTiles + anc_tile_capacity(p.max_anc);               // listed tiles
-    uint32_t* valid_s = reinterpret_cast<uint32_t*>(key_s + cap * kTileN);   // [cap]
-    uint32_t* spec_s = valid_s + ((cap + 3) & ~3);                           // [8] per-wave flags of the start-up
-    uint32_t* mask_s = spec_s + 8;                                           // [ancestor tiles][M], 16-byte aligned
+    // this workgroup's part of the block plan: header | ancestor keys | per 32 rows: leaf keys, mask words
+    const int anc_cap = anc_tile_capacity(p.max_anc);
+    const int common_words = kPlanHeaderWords + anc_cap * kTileN;
+    const int group_words = kTileN * (1 + anc_cap);
+    uint32_t* plan_s = reinterpret_cast<uint32_t*>(ring + stages * 2 * kTileElems);
+    uint32_t* group_s = plan_s + common_words;            // [kLeafTiles][group_words]
 
     // All kernel arguments are fetched by ONE batch of scalar loads.  Left to itself the compiler
     // loads each field just before its first use, which puts four dependent round trips to the
     // argument segment in front of the first memory request of the workgroup.
-    asm volatile("" ::"s"(p.q), "s"(p.k), "s"(p.v), "s"(p.o), "s"(p.lse), "s"(p.ancestor_idx), "s"(p.mask_bits),
-                 "s"(p.anc_count), "s"(p.leaf_idx), "s"(p.nq), "s"(p.nk), "s"(p.prefix), "s"(p.max_anc),
-                 "s"(p.mask_words), "s"(p.nb), "s"(p.heads_total), "s"(p.out_f32), "s"(p.scale_log2e), "s"(stages),
-                 "s"(early_leaf), "s"(sub_shift));
+    asm volatile("" ::"s"(p.q), "s"(p.k), "s"(p.v), "s"(p.o), "s"(p.lse), "s"(p.plan), "s"(p.key_shift),
+                 "s"(p.nq), "s"(p.nk), "s"(p.prefix), "s"(p.max_anc), "s"(p.nb), "s"(p.heads_total), "s"(p.out_f32),
+                 "s"(p.scale_log2e), "s"(stages), "s"(early_leaf), "s"(sub_shift));
 
     // Workgroup -> (slice, block), XCD-aware: every XCD gets whole (batch, head) slices, so all
     // query blocks of a slice share one L2 for the K/V rows they have in common.  The grid is
@@ -163,56 +163,37 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     const int ql = lane & 15;        // query (column of S^T / O^T) of this lane
     const int g = lane >> 4;         // which quarter of the rows of an accumulator tile
     const int row_in_block = qgroup * 16 + ql;
-    const int qrow = row_base + row_in_block;
 
     const T* qb = static_cast<const T*>(p.q) + (size_t)hz * p.nq * D;
     const T* kb = static_cast<const T*>(p.k) + (size_t)hz * p.nk * D;
     const T* vb = static_cast<const T*>(p.v) + (size_t)hz * p.nk * D;
 
-    // ---- start-up: everything that needs no metadata goes out before the metadata is read ----
-    // Loads and transfers retire in issue order.  The key lists go first (the longest chain hangs
-    // on them: sanitise, barrier, ancestor requests), then mask words, Q rows and the first leaf
-    // tiles.  The number of transfers issued after the mask words is a compile-time constant: the
-    // wait for the lists (and the mask words behind them) can then leave exactly those in flight.
-    // (the block's ancestor count: requested first, read when the key lists have arrived)
-    uint32_t anc_count_raw = 0u;
-    if (p.anc_count) anc_count_raw = global_read_b32(p.anc_count + j);
-    // Key lists: the block's M leaf slots, then its ancestor slots, kKeyBatch per thread and
-    // round.  Slots past the end of the lists re-read the last entry and are blanked below.
-    constexpr int kKeyBatch = 2;
-    auto load_ids = [&](int c0, u32x2 (&raw)[kKeyBatch]) {
-#pragma unroll
-        for (int i = 0; i < kKeyBatch; ++i) {
-            const int c = c0 + i * kThreads;
-            const int64_t* src = c < M ? p.leaf_idx + (size_t)row_base + c
-                                       : p.ancestor_idx + (size_t)j * p.max_anc + min(c - M, p.max_anc - 1);
-            raw[i] = global_read_b64(src);
-        }
-    };
-    auto ids_of = [&](int c0, u32x2 (&raw)[kKeyBatch], int64_t (&ids)[kKeyBatch]) {
-#pragma unroll
-        for (int i = 0; i < kKeyBatch; ++i) {
-            lds_tie(raw[i]);
-            const int c = c0 + i * kThreads;
-            ids[i] = c - M < p.max_anc ? (int64_t)(((uint64_t)raw[i][1] << 32) | raw[i][0]) : -1;
-        }
-    };
-    u32x2 leaf_raw = global_read_b64(p.leaf_idx + (size_t)row_base + row_in_block);
-    u32x2 first_raw[kKeyBatch];
-    load_ids(tid, first_raw);
-    // mask words: straight global->LDS copy, 16 bytes per lane, 1 KiB pieces dealt to the waves
+    // ---- start-up: every request that needs no metadata goes out together with the metadata ----
+    // Loads and transfers retire in issue order.  The block plan goes first (the ancestor requests
+    // hang on it), then the Q rows and, in a launch whose workgroups all run at once, the first
+    // leaf tiles.  The number of transfers issued after the plan is a compile-time constant: the
+    // wait for the plan can then leave exactly those in flight.
+    // The plan holds what a workgroup needs of the tree in the form it is used in: 32-bit K/V rows
+    // per tile slot (empty slots repeat a row), leaf validity, mask words per (ancestor tile, row).
+    // Record of block j: common part, then one group per 32 rows; this workgroup takes the
+    // common part and its own M/32 groups, which land next to each other in LDS.
+    // In a small launch (`early_leaf`) every wave copies the whole piece for itself (it is a few
+    // hundred bytes, all waves write the same values to the same place): a wave then depends on
+    // no other wave until the first tile is consumed.  Otherwise the waves share the copy and
+    // meet at a barrier.
     {
-        // source: [word][block_rows] words of block j, of which this workgroup takes M per word
-        const int chunks = p.mask_words * (M / 4);     // 16-byte pieces
-        const char* src = reinterpret_cast<const char*>(p.mask_bits) +
-                          ((size_t)j * p.mask_words * block_rows + (row_base - j * block_rows)) * 4;
-        for (int piece = wave; piece * 64 < chunks; piece += kWaves) {
+        const int block_groups = block_rows / kTileN;
+        const char* rec = reinterpret_cast<const char*>(p.plan) +
+                          (size_t)j * (size_t)(common_words + block_groups * group_words) * 4;
+        const int common_chunks = common_words / 4;                       // 16-byte pieces
+        const int chunks = common_chunks + kLeafTiles * (group_words / 4);
+        const uint32_t group_skip = (uint32_t)(((row_base - j * block_rows) / kTileN) * group_words * 4);
+        for (int piece = early_leaf ? 0 : wave; piece * 64 < chunks; piece += early_leaf ? 1 : kWaves) {
             const int c = piece * 64 + lane;
-            if (c < chunks)   // (uniform base + 32-bit lane offset: a block's mask words are a few KiB)
+            if (c < chunks)
                 __builtin_amdgcn_global_load_lds(
-                    (const void __attribute__((address_space(1)))*)(src + (size_t)(uint32_t)((c / (M / 4)) * block_rows * 4 +
-                                                                                             (c % (M / 4)) * 16)),
-                    (void __attribute__((address_space(3)))*)(reinterpret_cast<char*>(mask_s) + piece * 1024),
+                    (const void __attribute__((address_space(1)))*)(rec + (size_t)((uint32_t)c * 16u + (c >= common_chunks ? group_skip : 0u))),
+                    (void __attribute__((address_space(3)))*)(reinterpret_cast<char*>(plan_s) + piece * 1024),
                     16, 0, 0);
         }
     }
@@ -222,10 +203,10 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     const int dma_row = lane / kCpr, dma_slot = lane % kCpr;
     constexpr int kQDma = 16 / kRowsPerDma;
     static_assert(kQDma >= 1, "a transfer covers at most the wave's 16 rows");
-    // (a small grid has LDS to spare: Q then gets an area of its own behind the mask words, the
+    // (a small grid has LDS to spare: Q then gets an area of its own behind the plan, the
     // whole ring is free from the start and the fragments are read after the ancestor tiles have
     // been requested instead of in front of the first barrier)
-    T* qstage = early_leaf ? reinterpret_cast<T*>(mask_s + anc_tile_capacity(p.max_anc) * M) + wave * 16 * D
+    T* qstage = early_leaf ? reinterpret_cast<T*>(group_s + kLeafTiles * group_words) + wave * 16 * D
                            : ring + (size_t)stages * 2 * kTileElems - (kWaves - wave) * 16 * D;
 #pragma unroll
     for (int i = 0; i < kQDma; ++i) {
@@ -246,25 +227,27 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     // A lane's address is slice base (uniform) + a 32-bit byte offset: row * row pitch + the chunk
     // its slot holds.  The chunk offsets are fixed for the kernel's life (dma_anc / dma_leaf); a
     // request then costs one multiply-add per transfer.  (The launcher keeps slices below 4 GiB.)
-    uint32_t dma_anc[kDmaPerWave], dma_leaf[kDmaPerWave];
+    // (dma_flip = ancestor-tile offset XOR leaf-tile offset, applied under an all-ones / all-zeros
+    // word: a select between elements of two arrays makes the compiler address the arrays through a
+    // selected pointer, i.e. keep them in scratch memory, whose reloads share vmcnt with the ring)
+    uint32_t dma_leaf[kDmaPerWave], dma_flip[kDmaPerWave];
 #pragma unroll
     for (int i = 0; i < kDmaPerWave; ++i) {
         const int t2 = wave * kDmaPerWave + i;
         const int r = (t2 >> 1) * kRowsPerDma + dma_row;
         // V of a leaf tile is read row-wise like K (no transposing read), so it takes K's swizzle
         dma_leaf[i] = (uint32_t)k_chunk<D>(r, dma_slot) * 16u;
-        dma_anc[i] = (t2 & 1) ? (uint32_t)v16_chunk<D>(r, dma_slot) * 16u : dma_leaf[i];
+        dma_flip[i] = (t2 & 1) ? ((uint32_t)v16_chunk<D>(r, dma_slot) * 16u) ^ dma_leaf[i] : 0u;
     }
     auto issue_rows = [&](int t, int slot, const int (&rows)[kRowGroups]) {
         T* dst_tile = ring + slot * 2 * kTileElems;
-        const bool leaf_tile = t < kLeafTiles;
+        const uint32_t anc_tile = t < kLeafTiles ? 0u : 0xffffffffu;
 #pragma unroll
         for (int i = 0; i < kDmaPerWave; ++i) {
             const int t2 = wave * kDmaPerWave + i;
             const int u = t2 >> 1;
             const bool is_v = t2 & 1;
-            const uint32_t off = (uint32_t)rows[i >> 1] * (uint32_t)(D * sizeof(T)) +
-                                 (leaf_tile ? dma_leaf[i] : dma_anc[i]);
+            const uint32_t off = (uint32_t)rows[i >> 1] * (uint32_t)(D * sizeof(T)) + (dma_leaf[i] ^ (dma_flip[i] & anc_tile));
             const char* src = reinterpret_cast<const char*>(is_v ? vb : kb) + (size_t)off;
             __builtin_amdgcn_global_load_lds(
                 (const void __attribute__((address_space(1)))*)src,
@@ -290,54 +273,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         issue_rows(t, t, rows);
     }
 
-    // Sanitised key lists: the block's M leaf slots (tiles 0 .. kLeafTiles-1), then the ancestor
-    // slots.  An empty or out-of-range slot is given the row of the first valid key of its tile
-    // (row 0 if the tile has none): the transfer count per tile stays fixed, the slot's mask
-    // bits are cleared through valid_s, and the data it brings in is data the tile holds anyway.
-    auto store_keys = [&](int c0, const int64_t (&ids)[kKeyBatch]) {
-#pragma unroll
-        for (int i = 0; i < kKeyBatch; ++i) {
-            const int c = c0 + i * kThreads;
-            if (c < cap * kTileN) {
-                const bool ok = (uint64_t)ids[i] < (uint64_t)p.nk;   // 0 <= id < nk
-                const uint64_t vote = __ballot(ok);
-                const uint32_t lo = (uint32_t)vote, hi = (uint32_t)(vote >> 32);   // two tiles per wave
-                const int mine_id = ok ? (int)ids[i] : 0;
-                // first valid row of each tile: wave-uniform lane numbers, so plain lane reads.  A
-                // tile without a valid slot reads its last lane, which then holds row 0.
-                const int first_lo = __builtin_amdgcn_readlane(mine_id, __builtin_ctz(lo | 0x80000000u));
-                const int first_hi = __builtin_amdgcn_readlane(mine_id, 32 + __builtin_ctz(hi | 0x80000000u));
-                const uint32_t mine = lane < 32 ? lo : hi;
-                const int fallback = lane < 32 ? first_lo : first_hi;
-                lds_write_b32(lds_addr(key_s + c), ok ? (int)ids[i] : fallback);
-                if ((lane & 31) == 0) lds_write_b32(lds_addr(valid_s + (c >> 5)), mine);
-            }
-        }
-    };
-    // first batch and the leaf check: wait for the lists, leave the transfers behind them in flight
     const bool gathers = !(kDmaWaves < kWaves && wave >= kDmaWaves);
-    if (gathers && n_spec) wait_vmcnt<kQDma + kEarlyTiles * kDmaPerWave>();
-    else wait_vmcnt<kQDma>();
-    int64_t first_ids[kKeyBatch];
-    ids_of(tid, first_raw, first_ids);
-    lds_tie(leaf_raw);
-    const int64_t leaf64 = (int64_t)(((uint64_t)leaf_raw[1] << 32) | leaf_raw[0]);
-    store_keys(tid, first_ids);
-    const bool leaf_ok = tree && leaf64 >= 0 && leaf64 < p.nk;
-    {   // does any valid leaf slot name another row than the one requested above?
-        const bool other = leaf_ok && (row_in_block >> 5) < n_spec && leaf64 != (int64_t)p.prefix + qrow;
-        if (lane == 0) lds_write_b32(lds_addr(spec_s + wave), 0u);
-        if (other) lds_write_b32(lds_addr(spec_s + wave), 1u);
-    }
-    // ... further batches only for very long ancestor lists
-    for (int c0 = tid + kKeyBatch * kThreads; c0 < cap * kTileN; c0 += kKeyBatch * kThreads) {
-        u32x2 raw[kKeyBatch];
-        int64_t ids[kKeyBatch];
-        load_ids(c0, raw);
-        wait_vmcnt<0>();
-        ids_of(c0, raw, ids);
-        store_keys(c0, ids);
-    }
     // Q fragments: B operand of S^T = K.Q^T, lane holds Q[q][32s + 8g .. +7].  Only the leaf
     // tiles requested above were issued after the Q rows.
     Frag qf[kSteps];
@@ -354,9 +290,40 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
             qf[s] = __builtin_bit_cast(Frag, qraw[s]);
         }
     };
-    if (!early_leaf) read_q(0);   // Q sits in ring slots the gathers are about to take
-    lds_tie(anc_count_raw);
-    int n_anc = p.anc_count ? __builtin_amdgcn_readfirstlane((int)anc_count_raw) : p.max_anc;
+    if (early_leaf) {
+        // this wave's own copy of the plan has landed; the Q rows and leaf tiles stay in flight
+        if (gathers && n_spec) wait_vmcnt<kQDma + kEarlyTiles * kDmaPerWave>();
+        else wait_vmcnt<kQDma>();
+    } else {
+        read_q(0);        // Q sits in ring slots the gathers are about to take (waits for all of this wave's transfers)
+        ring_barrier();   // everybody's pieces of the plan have landed, everybody has read its Q rows
+    }
+    // From the plan: ancestor count, validity of this lane's own leaf slot and, after early leaf
+    // requests, whether any valid leaf slot names another row than the one requested (lane i looks
+    // at slot i of the tiles requested: every wave sees all of them and decides alike).
+    const int first_group = (row_base - j * block_rows) / kTileN;   // this workgroup's first group of 32 rows
+    bool leaf_ok, restart = false;
+    int n_anc;
+    {
+        uint32_t head = lds_read_b32(lds_addr(plan_s));
+        uint32_t my_valid = lds_read_b32(lds_addr(plan_s + kPlanLeafValid + first_group + (row_in_block >> 5)));
+        uint32_t spec_valid = 0u, spec_key = 0u;
+        const bool checks = lane < n_spec * kTileN;
+        if (checks) {
+            spec_valid = lds_read_b32(lds_addr(plan_s + kPlanLeafValid + first_group + (lane >> 5)));
+            spec_key = lds_read_b32(lds_addr(group_s + (lane >> 5) * group_words + (lane & 31)));
+        }
+        lds_wait();
+        lds_tie(head);
+        lds_tie(my_valid);
+        lds_tie(spec_valid);
+        lds_tie(spec_key);
+        n_anc = __builtin_amdgcn_readfirstlane((int)head);
+        leaf_ok = tree && ((my_valid >> (row_in_block & 31)) & 1u);
+        const bool other = checks && ((spec_valid >> (lane & 31)) & 1u) &&
+                           (int)spec_key + p.key_shift != p.prefix + row_base + lane;
+        restart = __ballot(other) != 0ull;
+    }
     n_anc = tree ? min(max(n_anc, 0), p.max_anc) : 0;
     const int listed_tiles = kLeafTiles + (n_anc + kTileN - 1) / kTileN;
     int prefix_first = 0, prefix_end = (p.prefix + kTileN - 1) / kTileN;   // this workgroup's prefix tiles
@@ -366,15 +333,16 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     }
     const int total_tiles = listed_tiles + prefix_end - prefix_first;
     const int prefix_shift = prefix_first - listed_tiles;   // list position t holds prefix tile t + prefix_shift
-    ring_barrier();
 
     auto issue = [&](int t, int slot) {
         if (kDmaWaves < kWaves && wave >= kDmaWaves) return;
         int rows[kRowGroups];
         if (kDShare || t < listed_tiles) {   // (head-dimension pairing is launched without a prefix)
+            const uint32_t* keys = t < kLeafTiles ? group_s + t * group_words
+                                                  : plan_s + kPlanHeaderWords + (t - kLeafTiles) * kTileN;
 #pragma unroll
-            for (int i = 0; i < kRowGroups; ++i)
-                rows[i] = key_s[t * kTileN + ((wave * kDmaPerWave) / 2 + i) * kRowsPerDma + dma_row];
+            for (int i = 0; i < kRowGroups; ++i)   // (the clamp keeps a plan made for more K/V rows from reaching past them)
+                rows[i] = min((int)keys[((wave * kDmaPerWave) / 2 + i) * kRowsPerDma + dma_row] + p.key_shift, p.nk - 1);
         } else {
 #pragma unroll
             for (int i = 0; i < kRowGroups; ++i)
@@ -428,25 +396,11 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         if (sl >= stages) sl -= stages;
         return ring + sl * 2 * kTileElems;
     };
-    {   // a leaf list that names other rows than the ones requested: start the ring over
-        const u32x4 f0 = lds_read_b128(lds_addr(spec_s)), f1 = lds_read_b128(lds_addr(spec_s + 4));
-        lds_wait();
-        u32x4 lo = f0, hi = f1;
-        lds_tie(lo);
-        lds_tie(hi);
-        uint32_t any = 0u;   // only the flags of waves that exist have been written
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const uint32_t a = lo[w], b = hi[w];
-            if (w < kWaves) any |= a;
-            if (w + 4 < kWaves) any |= b;
-        }
-        if (__builtin_amdgcn_readfirstlane(any) != 0u) {
-            wait_vmcnt<0>();
-            __syncthreads();
-            issued = consumed;
-            issue_slot = 0;
-        }
+    if (restart) {   // a leaf list that names other rows than the ones requested: start the ring over
+        wait_vmcnt<0>();
+        __syncthreads();
+        issued = consumed;
+        issue_slot = 0;
     }
     refill();
     if (early_leaf) read_q(issued);
@@ -517,6 +471,8 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     const int tr_r0 = 4 * g + (ql >> 2);   // this lane's key row for the transposing read
     const int tr_col = 4 * (ql & 3);       // head dim within the 16-row tile
     const uint32_t v_lane0 = (uint32_t)(tr_r0 * D + v16_chunk<D>(tr_r0, tr_col >> 3) * 8 + (tr_col & 7)) * 2;
+    // this row's mask words, one per ancestor tile (bits of empty slots are clear in the plan)
+    const uint32_t* my_mask = group_s + (row_in_block >> 5) * group_words + kTileN + (row_in_block & 31);
     while (consumed < total_tiles) {
         begin_step(kSplit);
         const int t = consumed + (kDShare ? 0 : split);
@@ -525,7 +481,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         end_step(kSplit);
         uint32_t word = 0u;
         if (t < listed_tiles) {
-            word = mask_s[(t - kLeafTiles) * M + row_in_block] & valid_s[t];
+            word = my_mask[(t - kLeafTiles) * kTileN];
         } else if (t < total_tiles) {
             const int left = p.prefix - (t + prefix_shift) * kTileN;
             word = left >= 32 ? 0xffffffffu : ((1u << left) - 1u);
@@ -859,7 +815,7 @@ int launch_d(const AttnParams& p, int head_dim, hipStream_t stream) {
 
 int launch_attention_mfma16(const AttnParams& p, int dtype, int head_dim, bool fast_pv, hipStream_t stream) {
     // the gathers address a (batch, head) slice of K or V with 32-bit byte offsets
-    if ((uint64_t)p.nk * (uint64_t)head_dim * 2u > 0xffffffffull) return FSTA_EUNSUPPORTED;
+    if ((uint64_t)p.nk * (uint64_t)head_dim * 2u > 0xffffffffull || !p.plan) return FSTA_EUNSUPPORTED;
     if (dtype == FSTA_F16) return launch_d<false, false>(p, head_dim, stream);
     if (fast_pv) return launch_d<true, false>(p, head_dim, stream);
     return launch_d<true, true>(p, head_dim, stream);

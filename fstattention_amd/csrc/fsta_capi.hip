@@ -76,11 +76,13 @@ extern "C" size_t fsta_attention_workspace_bytes(int32_t batch, int32_t heads, i
 extern "C" int fsta_attention_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                                   const int64_t* ancestor_idx, const uint32_t* mask_bits,
                                   const int32_t* anc_count, const int64_t* leaf_idx,
+                                  const uint32_t* block_plan, int32_t plan_key_shift,
                                   int32_t batch, int32_t heads, int32_t nq, int32_t nk,
                                   int32_t head_dim, int32_t dtype, int32_t out_dtype,
                                   int32_t block_m, int32_t max_ancestors, int32_t num_blocks,
                                   float sm_scale, uint32_t flags, void* stream) {
-    return fsta_attention_fwd_ws(q, k, v, o, lse, ancestor_idx, mask_bits, anc_count, leaf_idx, batch, heads, nq,
+    return fsta_attention_fwd_ws(q, k, v, o, lse, ancestor_idx, mask_bits, anc_count, leaf_idx, block_plan,
+                                 plan_key_shift, batch, heads, nq,
                                  nk, head_dim, dtype, out_dtype, block_m, max_ancestors, num_blocks, sm_scale,
                                  flags, nullptr, 0, stream);
 }
@@ -88,6 +90,7 @@ extern "C" int fsta_attention_fwd(const void* q, const void* k, const void* v, v
 extern "C" int fsta_attention_fwd_ws(const void* q, const void* k, const void* v, void* o, float* lse,
                                      const int64_t* ancestor_idx, const uint32_t* mask_bits,
                                      const int32_t* anc_count, const int64_t* leaf_idx,
+                                     const uint32_t* block_plan, int32_t plan_key_shift,
                                      int32_t batch, int32_t heads, int32_t nq, int32_t nk,
                                      int32_t head_dim, int32_t dtype, int32_t out_dtype,
                                      int32_t block_m, int32_t max_ancestors, int32_t num_blocks,
@@ -116,15 +119,24 @@ extern "C" int fsta_attention_fwd_ws(const void* q, const void* k, const void* v
     if (slices == 0 || nq == 0) return FSTA_OK;
     if (!q || !k || !v || !o || !ancestor_idx || !mask_bits || !leaf_idx)
         return fail(FSTA_EINVAL, "fsta_attention_fwd: null pointer");
-    // rows are moved 16 bytes at a time
-    if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
-         reinterpret_cast<uintptr_t>(o)) % 16 != 0)
+    // rows and plan records are moved 16 bytes at a time, list entries 8, mask words and counts 4
+    if (misaligned(q, 16) || misaligned(k, 16) || misaligned(v, 16) || misaligned(o, 16))
         return fail(FSTA_EINVAL, "fsta_attention_fwd: q, k, v and o must be 16-byte aligned");
+    if (misaligned(block_plan, 16))
+        return fail(FSTA_EINVAL, "fsta_attention_fwd: block_plan must be 16-byte aligned");
+    if (misaligned(ancestor_idx, 8) || misaligned(leaf_idx, 8))
+        return fail(FSTA_EINVAL, "fsta_attention_fwd: ancestor_idx and leaf_idx must be 8-byte aligned");
+    if (misaligned(mask_bits, 4) || misaligned(anc_count, 4) || misaligned(lse, 4))
+        return fail(FSTA_EINVAL, "fsta_attention_fwd: mask_bits, anc_count and lse must be 4-byte aligned");
+    if (block_plan && (plan_key_shift < 0 || plan_key_shift > nk))
+        return fail(FSTA_EINVAL, "fsta_attention_fwd: plan_key_shift=%d outside [0, nk=%d]", plan_key_shift, nk);
 
     AttnParams p;
     p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse;
     p.ancestor_idx = ancestor_idx; p.mask_bits = mask_bits; p.anc_count = anc_count;
     p.leaf_idx = leaf_idx;
+    p.plan = plan_block_size_ok(block_m) ? block_plan : nullptr;
+    p.key_shift = plan_key_shift;
     p.nq = nq; p.nk = nk; p.prefix = nk - nq;
     p.block_m = block_m; p.max_anc = max_ancestors; p.mask_words = fsta_mask_words(max_ancestors);
     p.nb = num_blocks;
@@ -135,7 +147,7 @@ extern "C" int fsta_attention_fwd_ws(const void* q, const void* k, const void* v
     p.share_tiles = (flags & FSTA_FLAG_SHARE_TILES) ? 1 : 0;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (workspace) {
+    if (workspace && p.plan) {
         int split_tiles = 0;
         const int splits = plan_key_splits(slices, nq, nk, head_dim, dtype, block_m, sm_scale, flags, &split_tiles);
         if (splits > 1 && workspace_bytes >= key_split_bytes(splits, slices, nq, head_dim)) {
@@ -156,8 +168,10 @@ extern "C" int fsta_attention_fwd_ws(const void* q, const void* k, const void* v
     // the matrix-core kernel takes row maxima before scaling, which needs a positive scale
     if (!(flags & FSTA_FLAG_GENERIC) && sm_scale > 0.f && mfma_supported(dtype, head_dim, block_m)) {
         const bool fast_pv = (flags & FSTA_FLAG_FAST_PV) != 0;
-        const int rc = (flags & FSTA_FLAG_WIDE_WAVES) ? launch_attention_mfma(p, dtype, head_dim, fast_pv, s)
-                                                      : launch_attention_mfma16(p, dtype, head_dim, fast_pv, s);
+        // (the kernel with 16 rows per wave reads the block plan only; it hands launches it cannot
+        // take on to the other matrix-core kernel itself)
+        const int rc = (flags & FSTA_FLAG_WIDE_WAVES) || !p.plan ? launch_attention_mfma(p, dtype, head_dim, fast_pv, s)
+                                                                 : launch_attention_mfma16(p, dtype, head_dim, fast_pv, s);
         // ancestor lists too long for the LDS-resident lists of these kernels: the scalar kernel
         // streams them and takes any length
         if (rc != FSTA_EUNSUPPORTED) return rc;

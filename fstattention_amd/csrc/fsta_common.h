@@ -12,6 +12,26 @@ namespace fsta {
 
 constexpr float kLog2e = 1.4426950408889634f;
 
+// Block plan (include/fsta.h, fsta_block_plan_bytes): per query block a record of 32-bit words,
+//   header [kPlanHeaderWords] | ancestor keys [32 * tiles] | per 32 rows: leaf keys [32], mask words [tiles][32]
+constexpr int kPlanHeaderWords = 8;   // [0] ancestor count, [4..7] leaf validity per 32 rows
+constexpr int kPlanLeafValid = 4;
+struct PlanLayout {
+    int tiles;          // ancestor tiles of 32 slots
+    int common_words;   // header + ancestor keys
+    int group_words;    // one group of 32 rows: leaf keys + mask words
+    int block_words;    // whole record
+};
+__host__ __device__ inline PlanLayout plan_layout(int block_m, int max_anc) {
+    PlanLayout l;
+    l.tiles = (max_anc + 31) / 32;
+    l.common_words = kPlanHeaderWords + 32 * l.tiles;
+    l.group_words = 32 * (1 + l.tiles);
+    l.block_words = l.common_words + (block_m / 32) * l.group_words;
+    return l;
+}
+inline bool plan_block_size_ok(int block_m) { return block_m == 32 || block_m == 64 || block_m == 128; }
+
 // Argument block of every attention kernel.  Plain data, passed by value.
 struct AttnParams {
     const void* q;
@@ -23,6 +43,8 @@ struct AttnParams {
     const uint32_t* mask_bits;    // [nb, mask_words, block_m]
     const int32_t* anc_count;     // [nb]
     const int64_t* leaf_idx;      // [nb, block_m]
+    const uint32_t* plan;         // block plan of the same lists, or null
+    int32_t key_shift;            // added to the plan's keys
     int32_t nq, nk, prefix;       // prefix = nk - nq
     int32_t block_m, max_anc, mask_words, nb;
     int32_t heads_total;          // batch * heads
@@ -36,6 +58,9 @@ struct AttnParams {
     float* part_o;
     float* part_lse;
 };
+
+// true when a non-null pointer is not a multiple of `bytes` (null pointers are judged elsewhere)
+inline bool misaligned(const void* ptr, unsigned bytes) { return reinterpret_cast<uintptr_t>(ptr) % bytes != 0; }
 
 // Records a message for fsta_last_error() and returns `code`.
 int fail(int code, const char* fmt, ...);

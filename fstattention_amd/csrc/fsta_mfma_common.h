@@ -127,6 +127,11 @@ __device__ __forceinline__ u32x4 lds_read_b128(uint32_t addr) {
     asm volatile("ds_read_b128 %0, %1" : "=v"(out) : "v"(addr) : "memory");
     return out;
 }
+__device__ __forceinline__ uint32_t lds_read_b32(uint32_t addr) {
+    uint32_t out;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(out) : "v"(addr) : "memory");
+    return out;
+}
 __device__ __forceinline__ u32x2 lds_read_b64(uint32_t addr) {
     u32x2 out;
     asm volatile("ds_read_b64 %0, %1" : "=v"(out) : "v"(addr) : "memory");

@@ -26,14 +26,14 @@ __global__ __launch_bounds__(kMaxThreads) void block_precompute_kernel(
     int64_t n_nodes, int64_t width, int block_m, int max_anc, int mask_words, int mutate, int staged,
     int64_t* __restrict__ ancestor_idx, uint8_t* __restrict__ ancestor_mask,
     int64_t* __restrict__ leaf_idx, uint32_t* __restrict__ mask_bits,
-    int32_t* __restrict__ anc_count, uint32_t* __restrict__ status) {
+    int32_t* __restrict__ anc_count, uint32_t* __restrict__ plan, uint32_t* __restrict__ status) {
     extern __shared__ uint32_t lds[];
     const int n_words = (int)((n_nodes + 31) >> 5);
     uint32_t* bitmap = lds;                                   // ancestor set of this block
     uint32_t* rank_base = bitmap + n_words;                   // set bits in lower words
     uint32_t* mbits = rank_base + n_words;                    // [mask_words][block_m]
     int32_t* lvl_s = reinterpret_cast<int32_t*>(mbits + (size_t)mask_words * block_m);  // [block_m]
-    uint32_t* misc = reinterpret_cast<uint32_t*>(lvl_s + block_m);   // [0] a -1 was seen, [2] total count
+    uint32_t* misc = reinterpret_cast<uint32_t*>(lvl_s + block_m);   // [0] a -1 was seen, [2] total count, [3] a listed ancestor
     int32_t* vals_s = reinterpret_cast<int32_t*>(misc + 4);          // [rows * width] when staged
 
     const int tid = threadIdx.x;
@@ -134,7 +134,11 @@ __global__ __launch_bounds__(kMaxThreads) void block_precompute_kernel(
     if (total > (uint32_t)max_anc) err |= FSTA_PRE_TOO_MANY_ANCESTORS;
     const int kept = (int)min(total, (uint32_t)max_anc);
 
-    // 3. ancestor_idx: ascending ids, left aligned, -1 padded (utils.py:112,120)
+    // 3. ancestor_idx: ascending ids, left aligned, -1 padded (utils.py:112,120); the block plan
+    //    receives the same ids as 32-bit keys
+    const PlanLayout layout = plan_layout(block_m, max_anc);
+    uint32_t* rec = plan ? plan + (size_t)j * layout.block_words : nullptr;
+    const uint32_t last_tile_first = kept > 0 ? (uint32_t)((kept - 1) & ~31) : 0xffffffffu;   // first slot of the last tile in use
     for (int c = kept + tid; c < max_anc; c += threads) ancestor_idx[(size_t)j * max_anc + c] = -1;
     for (int w = tid; w < n_words; w += threads) {
         uint32_t bits = bitmap[w];
@@ -142,7 +146,11 @@ __global__ __launch_bounds__(kMaxThreads) void block_precompute_kernel(
         while (bits) {
             const int b = __ffs(bits) - 1;
             bits &= bits - 1u;
-            if (r < (uint32_t)max_anc) ancestor_idx[(size_t)j * max_anc + r] = (int64_t)w * 32 + b;
+            if (r < (uint32_t)max_anc) {
+                ancestor_idx[(size_t)j * max_anc + r] = (int64_t)w * 32 + b;
+                if (rec) rec[kPlanHeaderWords + r] = (uint32_t)(w * 32 + b);
+                if (r == last_tile_first) misc[3] = (uint32_t)(w * 32 + b);
+            }
             ++r;
         }
     }
@@ -195,6 +203,31 @@ __global__ __launch_bounds__(kMaxThreads) void block_precompute_kernel(
         for (int e = tid; e < mask_words * block_m; e += threads)
             mask_bits[(size_t)j * mask_words * block_m + e] = mbits[e];
     }
+    if (rec) {
+        // Block plan: what the attention kernel would otherwise derive from the lists in every
+        // workgroup.  An empty slot repeats a row its tile holds anyway (the first key of the last
+        // ancestor tile in use, the first leaf of a group of 32 rows), so that every tile is
+        // gathered with the same number of requests; its mask bits are zero by construction.
+        const int tiles = layout.tiles, groups = block_m / 32;
+        const uint32_t spare = kept > 0 ? misc[3] : (uint32_t)lo;
+        for (int c = kept + tid; c < tiles * 32; c += threads) rec[kPlanHeaderWords + c] = spare;
+        if (tid == 0) rec[0] = (uint32_t)kept;
+        else if (tid < kPlanHeaderWords && (tid < kPlanLeafValid || tid - kPlanLeafValid >= groups)) rec[tid] = 0u;
+        if (tid < block_m) {   // (block_m <= 128: the first two waves)
+            const int64_t id = lo + tid;
+            const bool is_anc = id < n_nodes && ((bitmap[id >> 5] >> (id & 31)) & 1u);
+            const uint64_t vote = __ballot(!is_anc);
+            const uint32_t mine = (tid & 32) ? (uint32_t)(vote >> 32) : (uint32_t)vote;   // this group of 32 rows
+            const uint32_t first_leaf = mine ? (uint32_t)(lo + (tid & ~31) + __builtin_ctz(mine)) : (uint32_t)lo;
+            uint32_t* grp = rec + layout.common_words + (tid >> 5) * layout.group_words;
+            grp[tid & 31] = is_anc ? first_leaf : (uint32_t)id;
+            if ((tid & 31) == 0) rec[kPlanLeafValid + (tid >> 5)] = mine;
+        }
+        for (int e = tid; e < groups * tiles * 32; e += threads) {
+            const int g = e / (tiles * 32), rem = e - g * tiles * 32;   // rem = 32 * tile + row within the group
+            rec[layout.common_words + g * layout.group_words + 32 + rem] = mbits[(rem >> 5) * block_m + g * 32 + (rem & 31)];
+        }
+    }
     if (ancestor_mask) {
         // one byte per (row, ancestor slot); 8 slots of a row per store where the layout allows
         uint8_t* out = ancestor_mask + (size_t)j * block_m * max_anc;
@@ -227,11 +260,14 @@ __global__ __launch_bounds__(kMaxThreads) void block_precompute_kernel(
     if (err) atomicOr(status, err);
 }
 
+constexpr int kPackMaxTiles = 512;   // ancestor tiles a block plan written by pack_mask_kernel can have
+
 __global__ __launch_bounds__(kThreads) void pack_mask_kernel(
     const int64_t* __restrict__ ancestor_idx, const uint8_t* __restrict__ ancestor_mask,
-    int block_m, int max_anc, int mask_words, uint32_t* __restrict__ mask_bits,
-    int32_t* __restrict__ anc_count) {
+    const int64_t* __restrict__ leaf_idx, int block_m, int max_anc, int mask_words, int64_t key_limit,
+    uint32_t* __restrict__ mask_bits, int32_t* __restrict__ anc_count, uint32_t* __restrict__ plan) {
     __shared__ int last_valid;
+    __shared__ uint32_t tile_valid[kPackMaxTiles];   // plan only: slots of a tile whose id lies in [0, key_limit)
     const int tid = threadIdx.x;
     const int j = blockIdx.x;
     if (tid == 0) last_valid = -1;
@@ -241,6 +277,37 @@ __global__ __launch_bounds__(kThreads) void pack_mask_kernel(
     for (int c = tid; c < max_anc; c += kThreads)
         if (idx[c] >= 0) mine = c;
     if (mine >= 0) atomicMax(&last_valid, mine);
+    const PlanLayout layout = plan_layout(block_m, max_anc);
+    uint32_t* rec = plan ? plan + (size_t)j * layout.block_words : nullptr;
+    if (rec) {
+        // keys of the ancestor slots, a half-wave per tile of 32: an empty or out-of-range slot
+        // repeats the first valid key of its tile (row 0 if there is none)
+        for (int c0 = 0; c0 < layout.tiles * 32; c0 += kThreads) {
+            const int c = c0 + tid;
+            if (c < layout.tiles * 32) {
+                const int64_t id = c < max_anc ? idx[c] : -1;
+                const bool ok = id >= 0 && id < key_limit;
+                const uint64_t vote = __ballot(ok);
+                const uint32_t half = (tid & 32) ? (uint32_t)(vote >> 32) : (uint32_t)vote;
+                const uint32_t key = ok ? (uint32_t)id : 0u;
+                const uint32_t first = __shfl(key, (tid & 32) + __builtin_ctz(half | 0x80000000u), 64);
+                rec[kPlanHeaderWords + c] = ok ? key : first;
+                if ((tid & 31) == 0) tile_valid[c >> 5] = half;
+            }
+        }
+        if (tid < block_m) {   // leaf slots, a half-wave per group of 32 rows
+            const int64_t id = leaf_idx[(size_t)j * block_m + tid];
+            const bool ok = id >= 0 && id < key_limit;
+            const uint64_t vote = __ballot(ok);
+            const uint32_t half = (tid & 32) ? (uint32_t)(vote >> 32) : (uint32_t)vote;
+            const uint32_t key = ok ? (uint32_t)id : 0u;
+            const uint32_t first = __shfl(key, (tid & 32) + __builtin_ctz(half | 0x80000000u), 64);
+            rec[layout.common_words + (tid >> 5) * layout.group_words + (tid & 31)] = ok ? key : first;
+            if ((tid & 31) == 0) rec[kPlanLeafValid + (tid >> 5)] = half;
+        }
+        if (tid >= 1 && tid < kPlanHeaderWords && (tid < kPlanLeafValid || tid - kPlanLeafValid >= block_m / 32)) rec[tid] = 0u;
+    }
+    __syncthreads();
     const uint8_t* in = ancestor_mask + (size_t)j * block_m * max_anc;
     for (int e = tid; e < mask_words * block_m; e += kThreads) {
         const int w = e / block_m, r = e - w * block_m;
@@ -249,10 +316,13 @@ __global__ __launch_bounds__(kThreads) void pack_mask_kernel(
         const int c1 = min(c0 + 32, max_anc);
         for (int c = c0; c < c1; ++c)
             if (in[(size_t)r * max_anc + c] && idx[c] >= 0) bits |= 1u << (c - c0);
-        mask_bits[(size_t)j * mask_words * block_m + e] = bits;
+        if (mask_bits) mask_bits[(size_t)j * mask_words * block_m + e] = bits;
+        if (rec) rec[layout.common_words + (r >> 5) * layout.group_words + 32 + w * 32 + (r & 31)] = bits & tile_valid[w];
     }
-    __syncthreads();
-    if (tid == 0) anc_count[j] = last_valid + 1;
+    if (tid == 0) {
+        if (anc_count) anc_count[j] = last_valid + 1;
+        if (rec) rec[0] = (uint32_t)(last_valid + 1);
+    }
 }
 
 // `lds_nodes` > 0: the workgroup first copies parent[0 .. lds_nodes) into LDS as int32 (the walks to
@@ -362,7 +432,7 @@ extern "C" int fsta_precompute(int64_t* lineage, const int64_t* level_lookup, in
                                int64_t width, int32_t block_m, int32_t max_ancestors,
                                int32_t mutate_lineage, int64_t* ancestor_idx,
                                uint8_t* ancestor_mask, int64_t* leaf_idx, uint32_t* mask_bits,
-                               int32_t* anc_count, uint32_t* status, void* stream) {
+                               int32_t* anc_count, uint32_t* block_plan, uint32_t* status, void* stream) {
     if (n_nodes < 0 || width < 1 || block_m < 1 || max_ancestors < 1)
         return fail(FSTA_EINVAL, "fsta_precompute: n_nodes=%lld width=%lld block_m=%d max_ancestors=%d",
                     (long long)n_nodes, (long long)width, block_m, max_ancestors);
@@ -370,6 +440,14 @@ extern "C" int fsta_precompute(int64_t* lineage, const int64_t* level_lookup, in
     if (!lineage || !level_lookup || !ancestor_idx || !leaf_idx || !status)
         return fail(FSTA_EINVAL, "fsta_precompute: null pointer");
     if (block_m > 4096) return fail(FSTA_EUNSUPPORTED, "fsta_precompute: block_m=%d > 4096", block_m);
+    if (block_plan && !plan_block_size_ok(block_m))
+        return fail(FSTA_EINVAL, "fsta_precompute: a block plan needs block_m 32, 64 or 128 (got %d)", block_m);
+    if (block_plan && n_nodes + block_m > 0x7fffffff)
+        return fail(FSTA_EUNSUPPORTED, "fsta_precompute: block plan keys are 32-bit (n_nodes=%lld)", (long long)n_nodes);
+    if (misaligned(lineage, 8) || misaligned(level_lookup, 8) || misaligned(ancestor_idx, 8) || misaligned(leaf_idx, 8))
+        return fail(FSTA_EINVAL, "fsta_precompute: lineage, level_lookup, ancestor_idx and leaf_idx must be 8-byte aligned");
+    if (misaligned(mask_bits, 4) || misaligned(anc_count, 4) || misaligned(status, 4) || misaligned(block_plan, 16))
+        return fail(FSTA_EINVAL, "fsta_precompute: mask_bits, anc_count and status must be 4-byte aligned, block_plan 16-byte");
     const int mask_words = fsta_mask_words(max_ancestors);
     const int64_t n_words = (n_nodes + 31) >> 5;
     if ((int64_t)block_m * width > 0x7fffffff)
@@ -394,23 +472,42 @@ extern "C" int fsta_precompute(int64_t* lineage, const int64_t* level_lookup, in
     hipLaunchKernelGGL(block_precompute_kernel, dim3((unsigned)nb), dim3(threads), lds,
                        static_cast<hipStream_t>(stream), lineage, level_lookup, n_nodes, width,
                        block_m, max_ancestors, mask_words, mutate_lineage, staged, ancestor_idx,
-                       ancestor_mask, leaf_idx, mask_bits, anc_count, status);
+                       ancestor_mask, leaf_idx, mask_bits, anc_count, block_plan, status);
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
 }
 
-extern "C" int fsta_pack_mask(const int64_t* ancestor_idx, const uint8_t* ancestor_mask,
-                              int32_t num_blocks, int32_t block_m, int32_t max_ancestors,
-                              uint32_t* mask_bits, int32_t* anc_count, void* stream) {
+extern "C" size_t fsta_block_plan_bytes(int32_t num_blocks, int32_t block_m, int32_t max_ancestors) {
+    if (num_blocks <= 0 || max_ancestors < 1 || !plan_block_size_ok(block_m)) return 0;
+    return (size_t)num_blocks * (size_t)plan_layout(block_m, max_ancestors).block_words * sizeof(uint32_t);
+}
+
+extern "C" int fsta_pack_mask(const int64_t* ancestor_idx, const uint8_t* ancestor_mask, const int64_t* leaf_idx,
+                              int32_t num_blocks, int32_t block_m, int32_t max_ancestors, int64_t key_limit,
+                              uint32_t* mask_bits, int32_t* anc_count, uint32_t* block_plan, void* stream) {
     if (num_blocks < 0 || block_m < 1 || max_ancestors < 1)
         return fail(FSTA_EINVAL, "fsta_pack_mask: num_blocks=%d block_m=%d max_ancestors=%d",
                     num_blocks, block_m, max_ancestors);
     if (num_blocks == 0) return FSTA_OK;
-    if (!ancestor_idx || !ancestor_mask || !mask_bits || !anc_count)
+    if (!ancestor_idx || !ancestor_mask || (!block_plan && (!mask_bits || !anc_count)))
         return fail(FSTA_EINVAL, "fsta_pack_mask: null pointer");
+    if (block_plan) {
+        if (!leaf_idx) return fail(FSTA_EINVAL, "fsta_pack_mask: a block plan needs leaf_idx");
+        if (!plan_block_size_ok(block_m))
+            return fail(FSTA_EINVAL, "fsta_pack_mask: a block plan needs block_m 32, 64 or 128 (got %d)", block_m);
+        if (key_limit < 0 || key_limit > 0x7fffffff)
+            return fail(FSTA_EINVAL, "fsta_pack_mask: key_limit=%lld outside [0, 2^31)", (long long)key_limit);
+        if (fsta_mask_words(max_ancestors) > kPackMaxTiles)
+            return fail(FSTA_EUNSUPPORTED, "fsta_pack_mask: block plan with max_ancestors=%d > %d", max_ancestors,
+                        kPackMaxTiles * 32);
+    }
+    if (misaligned(ancestor_idx, 8) || misaligned(leaf_idx, 8))
+        return fail(FSTA_EINVAL, "fsta_pack_mask: ancestor_idx and leaf_idx must be 8-byte aligned");
+    if (misaligned(mask_bits, 4) || misaligned(anc_count, 4) || misaligned(block_plan, 16))
+        return fail(FSTA_EINVAL, "fsta_pack_mask: mask_bits and anc_count must be 4-byte aligned, block_plan 16-byte");
     hipLaunchKernelGGL(pack_mask_kernel, dim3(num_blocks), dim3(kThreads), 0,
-                       static_cast<hipStream_t>(stream), ancestor_idx, ancestor_mask, block_m,
-                       max_ancestors, fsta_mask_words(max_ancestors), mask_bits, anc_count);
+                       static_cast<hipStream_t>(stream), ancestor_idx, ancestor_mask, leaf_idx, block_m,
+                       max_ancestors, fsta_mask_words(max_ancestors), key_limit, mask_bits, anc_count, block_plan);
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
 }

@@ -11,7 +11,7 @@ from typing import Optional
 import torch
 
 from . import _lib
-from .attention import PackedTreeMask, _on_device, _stream_ptr
+from .attention import PackedTreeMask, _cache_key, _on_device, _stream_ptr
 
 
 def _raise_for_status(status: int, max_ancestors: int):
@@ -69,23 +69,26 @@ def create_fst_attention_kernel_inputs(lineage, level_lookup, block_m=64, max_an
     l_idx = torch.empty((nb, block_m), dtype=torch.int64, device=dev)
     bits = torch.empty((nb, words, block_m), dtype=torch.int32, device=dev)
     count = torch.empty((nb,), dtype=torch.int32, device=dev)
+    plan_bytes = lib.fsta_block_plan_bytes(nb, block_m, max_ancestors)
+    plan = torch.empty((plan_bytes // 4,), dtype=torch.int32, device=dev) if plan_bytes else None
     if status is None:
         status = torch.zeros((1,), dtype=torch.int32, device=dev)
     with _on_device(dev):
         _lib.check(lib.fsta_precompute(
             lin.data_ptr(), lvl.data_ptr(), n, width, block_m, max_ancestors, int(mutate_lineage),
             a_idx.data_ptr(), a_mask.data_ptr() if want_bool_mask else None, l_idx.data_ptr(),
-            bits.data_ptr(), count.data_ptr(), status.data_ptr(), _stream_ptr(dev)))
+            bits.data_ptr(), count.data_ptr(), plan.data_ptr() if plan is not None else None,
+            status.data_ptr(), _stream_ptr(dev)))
     if check:
         _raise_for_status(int(status.item()), max_ancestors)
     if mutate_lineage and lin.data_ptr() != lineage.data_ptr():
         lineage.copy_(lin)
-    packed = PackedTreeMask(bits, count, block_m, max_ancestors)
+    packed = PackedTreeMask(bits, count, block_m, max_ancestors, plan)
     if on_host:
         out = (a_idx.cpu(), a_mask.cpu() if want_bool_mask else packed, l_idx.cpu())
     else:
-        if want_bool_mask:
-            key = (a_mask._version, a_idx.data_ptr(), a_idx._version, tuple(a_mask.shape))
+        key = _cache_key(a_idx, a_mask, l_idx) if want_bool_mask else None
+        if key is not None:     # (tensors made in inference mode keep no edit counters: packed per call instead)
             a_mask._fsta_packed = (key, packed)
         out = (a_idx, a_mask if want_bool_mask else packed, l_idx)
     return out if check else out + (status,)

@@ -82,9 +82,6 @@ def parents_from_lineage(lineage, level_lookup) -> np.ndarray:
 
 
 # --------------------------------------------------------------------------- #
-# the reference's own benchmark tree
-# --------------------------------------------------------------------------- #
-# --------------------------------------------------------------------------- #
 # lineage-aware node order (the reference's open item, README.md:19-20)
 # --------------------------------------------------------------------------- #
 def subtree_sizes(parent) -> np.ndarray:
@@ -157,6 +154,9 @@ def renumber_parents(parent, perm):
     return new_parent, rank
 
 
+# --------------------------------------------------------------------------- #
+# the reference's own benchmark tree
+# --------------------------------------------------------------------------- #
 def _level_starts(depth: int, topk: int, left_weight_factor: float) -> np.ndarray:
     starts = np.zeros(depth + 2, dtype=np.int64)
     size = topk

@@ -21,7 +21,7 @@
 extern "C" {
 #endif
 
-#define FSTA_ABI_VERSION 1
+#define FSTA_ABI_VERSION 2
 
 /* element types of q/k/v/o */
 #define FSTA_F32  0
@@ -69,6 +69,25 @@ const char* fsta_last_error(void);
 int32_t fsta_mask_words(int32_t max_ancestors);
 
 /*
+ * Size in bytes of the block plan of a tree (0 when block_m is not 32, 64 or
+ * 128: the kernel that reads plans takes no other block size).  The plan is the
+ * same information as ancestor_idx / leaf_idx / mask_bits / anc_count in the
+ * form the matrix-core attention kernel consumes without any per-launch
+ * preparation: per query block a record of 32-bit words
+ *   [0] anc_count  [1..3] 0  [4..7] leaf validity, one word per 32 rows
+ *   [8 ..)  32 * T ancestor keys (T = ceil(max_ancestors / 32)): K/V row of
+ *           every slot; an empty slot repeats a valid row of the block
+ *   then per group of 32 query rows: 32 leaf keys (K/V row of each row's own
+ *           key, an empty slot repeats a valid row), then T x 32 mask words
+ *           (word t of row r: bit b = row r attends ancestor slot 32 t + b;
+ *           bits of empty slots are 0)
+ * Records are 16-byte aligned and follow each other block by block.  No
+ * counterpart in the reference, whose kernel re-reads the int64 lists and the
+ * byte mask in every program (fstattention.py:61-67).
+ */
+size_t fsta_block_plan_bytes(int32_t num_blocks, int32_t block_m, int32_t max_ancestors);
+
+/*
  * Per-block tree precompute on the GPU; replaces the host loop of
  * create_fst_attention_kernel_inputs (reference utils.py:104-129) and is
  * bit-exact with it:
@@ -76,35 +95,45 @@ int32_t fsta_mask_words(int32_t max_ancestors);
  *   ancestor_mask [num_blocks, block_m, max_ancestors]  bool   (utils.py:113,126-127)
  *   leaf_idx      [num_blocks, block_m]                 int64  (utils.py:114,121-122)
  * with num_blocks = ceil(n_nodes / block_m); ancestor_mask may be NULL when only
- * the packed form is wanted.  Extra outputs for the attention kernel (either
+ * the packed form is wanted.  Extra outputs for the attention kernels (each
  * may be NULL):
  *   mask_bits     [num_blocks, fsta_mask_words(A), block_m] uint32, bit b of
  *                 word w of row r = ancestor_mask[j, r, 32*w + b]
  *   anc_count     [num_blocks] int32, number of valid entries of ancestor_idx[j]
+ *   block_plan    fsta_block_plan_bytes(num_blocks, block_m, A) bytes, 16-byte
+ *                 aligned (block_m 32, 64 or 128 only, else it must be NULL)
  * lineage [n_nodes, width] int64 and level_lookup [n_nodes] int64 follow the
  * layout of utils.py:43-44,66-75.  With mutate_lineage != 0 each node id is
  * written into its own level column of `lineage`, as utils.py:124-125 does to
  * the caller's tensor.  `status` (one uint32, must be zero on entry) receives
  * FSTA_PRE_* bits; where the reference raises (utils.py:120) the bit
  * FSTA_PRE_TOO_MANY_ANCESTORS is set and the surplus ancestors are dropped.
+ * Alignment: lineage, level_lookup, ancestor_idx, leaf_idx 8 bytes; mask_bits,
+ * anc_count, status 4 bytes.
  */
 int fsta_precompute(int64_t* lineage, const int64_t* level_lookup,
                     int64_t n_nodes, int64_t width,
                     int32_t block_m, int32_t max_ancestors, int32_t mutate_lineage,
                     int64_t* ancestor_idx, uint8_t* ancestor_mask, int64_t* leaf_idx,
-                    uint32_t* mask_bits, int32_t* anc_count, uint32_t* status,
-                    void* stream);
+                    uint32_t* mask_bits, int32_t* anc_count, uint32_t* block_plan,
+                    uint32_t* status, void* stream);
 
 /*
  * Packs a boolean ancestor_mask [num_blocks, block_m, max_ancestors] (one byte
  * per entry, the tensor utils.py:104-129 returns) into mask_bits (layout above)
  * and counts, per block, the leading slots of ancestor_idx up to and including
  * the last non-negative one into anc_count.  Bits of slots whose ancestor_idx
- * is negative are cleared.
+ * is negative are cleared.  With block_plan != NULL (then leaf_idx
+ * [num_blocks, block_m] int64 is required, block_m 32, 64 or 128) the block
+ * plan of these lists is written as well; ids outside [0, key_limit) count as
+ * empty slots there (key_limit = number of K/V rows the lists address).
+ * Alignment: ancestor_idx, leaf_idx 8 bytes; mask_bits, anc_count 4 bytes;
+ * block_plan 16 bytes.
  */
 int fsta_pack_mask(const int64_t* ancestor_idx, const uint8_t* ancestor_mask,
-                   int32_t num_blocks, int32_t block_m, int32_t max_ancestors,
-                   uint32_t* mask_bits, int32_t* anc_count, void* stream);
+                   const int64_t* leaf_idx,
+                   int32_t num_blocks, int32_t block_m, int32_t max_ancestors, int64_t key_limit,
+                   uint32_t* mask_bits, int32_t* anc_count, uint32_t* block_plan, void* stream);
 
 /*
  * Fused sparse tree attention forward; replaces fst_attention/_fwd_kernel
@@ -123,7 +152,16 @@ int fsta_pack_mask(const int64_t* ancestor_idx, const uint8_t* ancestor_mask,
  * num_blocks must equal ceil(nq / block_m).  A row that attends to nothing
  * gets o = 0 and lse = -inf.
  * head_dim in {16,32,64,128}; block_m in {16,32,64,128}; max_ancestors >= 1.
- * q, k, v and o must be 16-byte aligned (rows are moved 16 bytes at a time).
+ * block_plan (may be NULL): the block plan of the same lists, as written by
+ * fsta_precompute or fsta_pack_mask with these block_m / max_ancestors;
+ * plan_key_shift is added to the plan's keys (the caller has added it to the
+ * valid entries of ancestor_idx and leaf_idx since the plan was made, e.g. the
+ * prefix length, fstattention.py:211-212).  The fastest kernel (16-bit types,
+ * head_dim >= 32, block_m >= 32) reads the plan only; without a plan a slower
+ * matrix-core kernel reads the lists themselves.  With a plan, the lists are
+ * still read by the kernels that serve the shapes the fast one does not take.
+ * Alignment: q, k, v, o and block_plan 16 bytes (rows are moved 16 bytes at a
+ * time); ancestor_idx and leaf_idx 8 bytes; mask_bits, anc_count and lse 4 bytes.
  * batch * heads <= 65535.  The matrix-core kernels address one (batch, head)
  * slice of K or V with 32-bit byte offsets: slices of 4 GiB and more
  * (nk * head_dim * 2 bytes) are served by the slower vector-ALU kernel.
@@ -131,6 +169,7 @@ int fsta_pack_mask(const int64_t* ancestor_idx, const uint8_t* ancestor_mask,
 int fsta_attention_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                        const int64_t* ancestor_idx, const uint32_t* mask_bits,
                        const int32_t* anc_count, const int64_t* leaf_idx,
+                       const uint32_t* block_plan, int32_t plan_key_shift,
                        int32_t batch, int32_t heads, int32_t nq, int32_t nk, int32_t head_dim,
                        int32_t dtype, int32_t out_dtype,
                        int32_t block_m, int32_t max_ancestors, int32_t num_blocks,
@@ -161,6 +200,7 @@ size_t fsta_attention_workspace_bytes(int32_t batch, int32_t heads, int32_t nq, 
 int fsta_attention_fwd_ws(const void* q, const void* k, const void* v, void* o, float* lse,
                           const int64_t* ancestor_idx, const uint32_t* mask_bits,
                           const int32_t* anc_count, const int64_t* leaf_idx,
+                          const uint32_t* block_plan, int32_t plan_key_shift,
                           int32_t batch, int32_t heads, int32_t nq, int32_t nk, int32_t head_dim,
                           int32_t dtype, int32_t out_dtype,
                           int32_t block_m, int32_t max_ancestors, int32_t num_blocks,

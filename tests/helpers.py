@@ -53,3 +53,37 @@ def assert_close(got, want, dtype, what=""):
     assert not bad.any(), (f"{what}: {int(bad.sum())} of {bad.numel()} elements outside "
                            f"atol=rtol={tol}; max err {float(err.max()):.3e}")
     return float(err.max())
+
+
+def expected_plan(a_idx, a_mask, l_idx, key_limit=None):
+    """The block plan (layout of include/fsta.h) of three index tensors (numpy), written from
+    their definition: (words uint32 [NB, block_words], care bool of the same shape).  `care` is
+    False on the keys of empty slots, which may repeat any row."""
+    nb, m, a = a_mask.shape
+    tiles, groups = (a + 31) // 32, m // 32
+    common = 8 + 32 * tiles
+    group = 32 * (1 + tiles)
+    words = np.zeros((nb, common + groups * group), dtype=np.uint32)
+    care = np.ones(words.shape, dtype=bool)
+    limit = 2 ** 31 - 1 if key_limit is None else key_limit
+    for j in range(nb):
+        valid_a = (a_idx[j] >= 0) & (a_idx[j] < limit)
+        words[j, 0] = np.flatnonzero(a_idx[j] >= 0).max(initial=-1) + 1
+        for c in range(32 * tiles):
+            if c < a and valid_a[c]:
+                words[j, 8 + c] = a_idx[j, c]
+            else:
+                care[j, 8 + c] = False
+        for r in range(m):
+            g, r5 = divmod(r, 32)
+            base = common + g * group
+            ok = 0 <= l_idx[j, r] < limit
+            if ok:
+                words[j, base + r5] = l_idx[j, r]
+                words[j, 4 + g] |= np.uint32(1 << r5)
+            else:
+                care[j, base + r5] = False
+            for c in range(a):
+                if a_mask[j, r, c] and valid_a[c]:
+                    words[j, base + 32 + (c // 32) * 32 + r5] |= np.uint32(1 << (c % 32))
+    return words, care

@@ -47,7 +47,7 @@ def test_header_is_plain_c_and_a_c_program_links(tmp_path):
         "    if (fsta_abi_version() != FSTA_ABI_VERSION) return 1;\n"
         "    if (fsta_mask_words(80) != 3) return 2;\n"
         "    /* rejected on the host, before any GPU work: head_dim 48 is not supported */\n"
-        "    int rc = fsta_attention_fwd(0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 1, 64, 64, 48, FSTA_BF16, FSTA_BF16,\n"
+        "    int rc = fsta_attention_fwd(0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 1, 64, 64, 48, FSTA_BF16, FSTA_BF16,\n"
         "                                64, 64, 1, 0.125f, 0, 0);\n"
         "    if (rc == FSTA_OK || strlen(fsta_last_error()) == 0) return 3;\n"
         '    printf("ok\\n");\n    return 0;\n}\n')
@@ -81,25 +81,49 @@ def test_argument_validation_happens_before_any_gpu_work():
     assert lib.fsta_abi_version() == _lib.ABI_VERSION
     assert lib.fsta_mask_words(1) == 1 and lib.fsta_mask_words(32) == 1 and lib.fsta_mask_words(33) == 2
     # every call below is rejected on its arguments; nothing is launched
-    bad_dtype = lib.fsta_attention_fwd(None, None, None, None, None, None, None, None, None,
+    bad_dtype = lib.fsta_attention_fwd(None, None, None, None, None, None, None, None, None, None, 0,
                                        1, 1, 16, 16, 64, 7, 7, 16, 8, 1, 1.0, 0, None)
     assert bad_dtype == _lib.EINVAL and b"dtype" in lib.fsta_last_error()
-    bad_dim = lib.fsta_attention_fwd(None, None, None, None, None, None, None, None, None,
+    bad_dim = lib.fsta_attention_fwd(None, None, None, None, None, None, None, None, None, None, 0,
                                      1, 1, 16, 16, 48, _lib.F16, _lib.F16, 16, 8, 1, 1.0, 0, None)
     assert bad_dim == _lib.EUNSUPPORTED and b"head_dim" in lib.fsta_last_error()
-    short_k = lib.fsta_attention_fwd(None, None, None, None, None, None, None, None, None,
+    short_k = lib.fsta_attention_fwd(None, None, None, None, None, None, None, None, None, None, 0,
                                      1, 1, 16, 8, 64, _lib.F16, _lib.F16, 16, 8, 1, 1.0, 0, None)
     assert short_k == _lib.EINVAL
-    blocks = lib.fsta_attention_fwd(None, None, None, None, None, None, None, None, None,
+    blocks = lib.fsta_attention_fwd(None, None, None, None, None, None, None, None, None, None, 0,
                                     1, 1, 40, 40, 64, _lib.F16, _lib.F16, 16, 8, 2, 1.0, 0, None)
     assert blocks == _lib.EINVAL and b"num_blocks" in lib.fsta_last_error()
-    null_ptr = lib.fsta_attention_fwd(None, None, None, None, None, None, None, None, None,
+    null_ptr = lib.fsta_attention_fwd(None, None, None, None, None, None, None, None, None, None, 0,
                                       1, 1, 16, 16, 64, _lib.F16, _lib.F16, 16, 8, 1, 1.0, 0, None)
     assert null_ptr == _lib.EINVAL and b"null" in lib.fsta_last_error()
-    assert lib.fsta_precompute(None, None, 10, 0, 4, 4, 0, None, None, None, None, None, None, None) == _lib.EINVAL
-    assert lib.fsta_precompute(None, None, 0, 1, 4, 4, 0, None, None, None, None, None, None, None) == _lib.OK
-    assert lib.fsta_pack_mask(None, None, 0, 16, 8, None, None, None) == _lib.OK
-    assert lib.fsta_pack_mask(None, None, 2, 16, 0, None, None, None) == _lib.EINVAL
+    # pointer alignment: rows and plan records move 16 bytes at a time, list entries 8, words 4
+    ok = dict(q=256, k=256, v=256, o=256, lse=256, a=256, bits=256, cnt=256, leaf=256, plan=256)
+
+    def attn(**ptr):
+        a = dict(ok, **ptr)
+        return lib.fsta_attention_fwd(a["q"], a["k"], a["v"], a["o"], a["lse"], a["a"], a["bits"], a["cnt"], a["leaf"],
+                                      a["plan"], 0, 1, 1, 64, 64, 64, _lib.BF16, _lib.BF16, 64, 32, 1, 0.125, 0, None)
+    for name, off, word in (("q", 8, b"16-byte"), ("k", 8, b"16-byte"), ("v", 4, b"16-byte"), ("o", 8, b"16-byte"),
+                            ("plan", 8, b"block_plan"), ("a", 4, b"8-byte"), ("leaf", 4, b"8-byte"),
+                            ("bits", 2, b"4-byte"), ("cnt", 2, b"4-byte"), ("lse", 2, b"4-byte")):
+        assert attn(**{name: 256 + off}) == _lib.EINVAL and word in lib.fsta_last_error(), name
+    assert lib.fsta_attention_fwd(256, 256, 256, 256, None, 256, 256, 256, 256, 256, -1, 1, 1, 64, 64, 64, _lib.BF16,
+                                  _lib.BF16, 64, 32, 1, 0.125, 0, None) == _lib.EINVAL      # negative key shift
+    assert lib.fsta_precompute(256, 256, 64, 4, 64, 32, 0, 260, None, 256, None, None, None, 256, None) == _lib.EINVAL
+    assert b"8-byte" in lib.fsta_last_error()
+    assert lib.fsta_precompute(256, 256, 64, 4, 64, 32, 0, 256, None, 256, 258, None, None, 256, None) == _lib.EINVAL
+    assert lib.fsta_precompute(256, 256, 64, 4, 64, 32, 0, 256, None, 256, None, None, 264, 256, None) == _lib.EINVAL
+    assert lib.fsta_precompute(256, 256, 64, 4, 16, 32, 0, 256, None, 256, None, None, 256, 256, None) == _lib.EINVAL
+    assert b"block plan" in lib.fsta_last_error()       # block sizes of the plan: 32, 64, 128
+    assert lib.fsta_pack_mask(260, 256, None, 2, 64, 32, 0, 256, 256, None, None) == _lib.EINVAL
+    assert lib.fsta_pack_mask(256, 256, None, 2, 64, 32, 0, 256, 256, 256, None) == _lib.EINVAL     # plan without leaf_idx
+    assert lib.fsta_pack_mask(256, 256, 256, 2, 64, 32, 64, 256, 256, 264, None) == _lib.EINVAL     # plan alignment
+    assert lib.fsta_block_plan_bytes(4, 64, 64) == 4 * (8 + 64 + 2 * (32 + 64)) * 4
+    assert lib.fsta_block_plan_bytes(4, 16, 64) == 0 and lib.fsta_block_plan_bytes(0, 64, 64) == 0
+    assert lib.fsta_precompute(None, None, 10, 0, 4, 4, 0, None, None, None, None, None, None, None, None) == _lib.EINVAL
+    assert lib.fsta_precompute(None, None, 0, 1, 4, 4, 0, None, None, None, None, None, None, None, None) == _lib.OK
+    assert lib.fsta_pack_mask(None, None, None, 0, 16, 8, 0, None, None, None, None) == _lib.OK
+    assert lib.fsta_pack_mask(None, None, None, 2, 16, 0, 0, None, None, None, None) == _lib.EINVAL
     assert lib.fsta_lineage_from_parents(None, 5, 0, None, None, None, None) == _lib.EINVAL
     assert lib.fsta_dfs_order(None, -1, 0, None, None, None, None, None) == _lib.EINVAL
     assert lib.fsta_dfs_order(None, 1 << 20, 0, None, None, None, None, None) == _lib.EUNSUPPORTED
@@ -149,11 +173,11 @@ def test_workspace_planning_is_host_arithmetic():
     assert size(0, 32, 256, 512, 128, _lib.BF16, 64, 64, 0.1, 0) == 0
     assert size(1, 32, 256, 100, 128, _lib.BF16, 64, 64, 0.1, 0) == 0
     # the workspace variant validates like the plain one, and wants an aligned workspace
-    bad = lib.fsta_attention_fwd_ws(None, None, None, None, None, None, None, None, None,
+    bad = lib.fsta_attention_fwd_ws(None, None, None, None, None, None, None, None, None, None, 0,
                                     1, 1, 16, 16, 64, 7, 7, 16, 8, 1, 1.0, 0, None, 0, None)
     assert bad == _lib.EINVAL and b"dtype" in lib.fsta_last_error()
     need = size(1, 32, 256, 256 + 16384, 128, _lib.BF16, 64, 64, 0.1, 0)
-    odd = lib.fsta_attention_fwd_ws(8, 8, 8, 8, None, 8, 8, None, 8, 1, 32, 256, 256 + 16384, 128, _lib.BF16,
+    odd = lib.fsta_attention_fwd_ws(16, 16, 16, 16, None, 8, 8, None, 8, 16, 0, 1, 32, 256, 256 + 16384, 128, _lib.BF16,
                                     _lib.BF16, 64, 64, 4, 0.1, 0, 4100, need, None)
     assert odd == _lib.EINVAL and b"aligned" in lib.fsta_last_error()
 

@@ -232,14 +232,15 @@ def test_key_runs_native_output_type_and_workspace_contract():
                                               _lib.flag_key_splits(1)) == 0
     assert lib.fsta_attention_workspace_bytes(1, h, nq, nq + prefix, d, _DTYPES[torch.float32], m, max_anc,
                                               scale, 0) == 0
-    packed = _packed_for(ad, md)
+    packed = _packed_for(ad, md, ld, nq + prefix)
     outs = []
     for work_bytes in (0, need - 1, need):
         work = torch.empty((max(work_bytes, 1),), dtype=torch.uint8, device="cuda")
         o32 = torch.empty(q.shape, dtype=torch.float32, device="cuda")
         _lib.check(lib.fsta_attention_fwd_ws(
             qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o32.data_ptr(), None, ad.data_ptr(),
-            packed.mask_bits.data_ptr(), packed.anc_count.data_ptr(), ld.data_ptr(), 1, h, nq, nq + prefix, d,
+            packed.mask_bits.data_ptr(), packed.anc_count.data_ptr(), ld.data_ptr(), packed.plan.data_ptr(),
+            packed.key_shift, 1, h, nq, nq + prefix, d,
             code, _DTYPES[torch.float32], m, max_anc, a_idx.shape[0], scale, 0,
             work.data_ptr() if work_bytes else None, work_bytes, torch.cuda.current_stream().cuda_stream))
         assert_close(o32, want, torch.bfloat16, f"workspace of {work_bytes} bytes")
@@ -369,6 +370,99 @@ def test_ancestor_slots_with_holes_and_out_of_range_ids_are_skipped():
         o = fst_attention(q.cuda(), k.cuda(), v.cuda(), wide_idx.cuda(), wide_mask.cuda(), l_idx.cuda(),
                           0.2, BLOCK_M=32, MAX_ANCESTORS=2 * max_anc, generic=generic)
         assert_close(o, want, torch.float32, "holes")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("block_m,heads", [(32, 2), (64, 40), (128, 3)])
+def test_holes_and_out_of_range_ids_in_the_block_plan(block_m, heads, dtype):
+    """The same malformed lists through the matrix-core kernel, whose block plan is made from them:
+    empty slots between valid ones, ids past the end of K with their mask bits set, leaf slots past
+    the end of K (small and large launches)."""
+    n = 3 * block_m
+    parent = trees.random_recursive_parents(n, 9, window=24)
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(parent, block_m, multiple=8)
+    nb = a_idx.shape[0]
+    wide_idx = torch.full((nb, 2 * max_anc), -1, dtype=torch.int64)
+    wide_mask = torch.zeros((nb, block_m, 2 * max_anc), dtype=torch.bool)
+    wide_idx[:, 1::2] = a_idx
+    wide_mask[:, :, 1::2] = a_mask
+    wide_idx[:, 0::4] = 10 ** 6
+    wide_mask[:, :, 0::2] = True
+    q, k, v = rand_qkv(1, heads, n, n, 64, dtype, 3)
+    want, _ = dense_oracle(q, k, v, parent, 0.2)
+    o = fst_attention(q.cuda(), k.cuda(), v.cuda(), wide_idx.cuda(), wide_mask.cuda(), l_idx.cuda(),
+                      0.2, BLOCK_M=block_m, MAX_ANCESTORS=2 * max_anc, out_dtype=torch.float32)
+    assert_close(o, want, dtype, "holes in the plan")
+    # a leaf slot past the end of K is an empty slot: rows that are nobody's ancestor then see nothing else
+    l_bad = l_idx.clone()
+    l_bad[l_bad >= 0] += 10 ** 6
+    o, lse = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_bad.cuda(), 0.2,
+                           BLOCK_M=block_m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32, return_lse=True)
+    mask = tp.dense_tree_mask(parent)
+    mask[np.arange(n), np.arange(n)] &= (l_idx.flatten()[:n] < 0).numpy()      # leaves lose their own key
+    want, _ = da_dense(q, k, v, mask, 0, 0.2)
+    want = torch.nan_to_num(want, nan=0.0)                                      # roots now see nothing: 0
+    assert_close(o, want, dtype, "leaf slots past the end of K")
+
+
+def test_packed_inputs_follow_a_prefix_shift_and_inference_mode():
+    """Kernel inputs made on the GPU as packed inputs (no bool mask), moved behind a shared prefix with
+    shift_for_prefix; the same calls under torch.inference_mode(), where tensors keep no version
+    counters and the bool mask is packed on every call."""
+    cfg = trees.config(2)
+    prefix, m, d, h = 96, cfg.block_m, 64, 3
+    parent = cfg.parent
+    lineage, level = trees.lineage_from_parents(parent)
+    max_anc = trees.required_max_ancestors(parent, m, 16)
+    n = len(parent)
+    q, k, v = rand_qkv(1, h, n, n + prefix, d, torch.bfloat16, 31)
+    scale = 0.125
+    want, _ = dense_oracle(q, k, v, parent, scale, prefix=prefix)
+    want0, _ = dense_oracle(q, k[:, :, prefix:], v[:, :, prefix:], parent, scale)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    for inference in (False, True):
+        with torch.inference_mode(inference):
+            a_idx, packed, l_idx = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), m, max_anc,
+                                                                      want_bool_mask=False)
+            assert packed.plan is not None and packed.key_shift == 0
+            o = fst_attention(qd, kd[:, :, prefix:].contiguous(), vd[:, :, prefix:].contiguous(), a_idx, packed, l_idx,
+                              scale, BLOCK_M=m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32)
+            assert_close(o, want0, torch.bfloat16, f"packed inputs, inference={inference}")
+            a_sh, l_sh, packed_sh = shift_for_prefix(a_idx, l_idx, prefix, packed)
+            assert packed_sh.key_shift == prefix
+            o = fst_attention(qd, kd, vd, a_sh, packed_sh, l_sh, scale, BLOCK_M=m, MAX_ANCESTORS=max_anc,
+                              out_dtype=torch.float32)
+            assert_close(o, want, torch.bfloat16, f"packed inputs behind a prefix, inference={inference}")
+            # bool mask: packed by fst_attention itself (kept on the tensor outside inference mode)
+            a_idx, a_mask, l_idx = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), m, max_anc)
+            assert hasattr(a_mask, "_fsta_packed") != inference
+            a_sh, l_sh = shift_for_prefix(a_idx, l_idx, prefix)
+            for _ in range(2):
+                o = fst_attention(qd, kd, vd, a_sh, a_mask, l_sh, scale, BLOCK_M=m, MAX_ANCESTORS=max_anc,
+                                  out_dtype=torch.float32)
+                assert_close(o, want, torch.bfloat16, f"bool mask behind a prefix, inference={inference}")
+
+
+def test_c_caller_without_a_block_plan_gets_the_list_reading_kernel():
+    """fsta_attention_fwd with block_plan = NULL: the lists themselves are read (slower matrix-core kernel)."""
+    from fstattention_amd import _lib
+    from fstattention_amd.attention import _DTYPES, pack_tree_mask
+    lib = _lib.load()
+    cfg = trees.config(2)
+    m, d, h = cfg.block_m, 128, 2
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(cfg.parent, m)
+    nq = a_idx.shape[0] * m
+    q, k, v = rand_qkv(1, h, nq, nq, d, torch.bfloat16, 5)
+    want, _ = dense_oracle(q, k, v, cfg.parent, 0.1, nq_pad=nq - len(cfg.parent))
+    qd, kd, vd, ad, md, ld = (t.cuda() for t in (q, k, v, a_idx, a_mask, l_idx))
+    packed = pack_tree_mask(ad, md)
+    assert packed.plan is None
+    o32 = torch.empty(q.shape, dtype=torch.float32, device="cuda")
+    _lib.check(lib.fsta_attention_fwd(
+        qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o32.data_ptr(), None, ad.data_ptr(), packed.mask_bits.data_ptr(),
+        packed.anc_count.data_ptr(), ld.data_ptr(), None, 0, 1, h, nq, nq, d, _DTYPES[torch.bfloat16],
+        _DTYPES[torch.float32], m, max_anc, a_idx.shape[0], 0.1, 0, torch.cuda.current_stream().cuda_stream))
+    assert_close(o32, want, torch.bfloat16, "no plan")
 
 
 @pytest.mark.parametrize("block_m,prefix,variant", [(32, 0, "default"), (64, 0, "default"), (128, 0, "default"),

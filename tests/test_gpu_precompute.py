@@ -130,6 +130,32 @@ def test_packed_mask_matches_bool_mask():
     np.testing.assert_array_equal(repacked.anc_count.cpu().numpy(), (a_idx.cpu().numpy() >= 0).sum(1))
 
 
+@pytest.mark.parametrize("block_m,n,window", [(32, 200, 16), (64, 500, 40), (128, 1000, 64), (64, 70, None), (128, 100, 3)])
+def test_block_plan_matches_the_lists(block_m, n, window):
+    """The kernel-ready record the precompute writes beside the three reference tensors (and the one
+    the packing entry point makes from them) holds exactly what they say; empty slots may repeat any
+    K/V row that exists, their mask bits are clear."""
+    from helpers import expected_plan
+    parent = trees.random_recursive_parents(n, 11 + n, window)
+    lineage, level = trees.lineage_from_parents(parent)
+    max_anc = trees.required_max_ancestors(parent, block_m, 16)
+    a_idx, a_mask, l_idx = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), block_m, max_anc)
+    made = a_mask._fsta_packed[1]
+    nb = a_idx.shape[0]
+    want, care = expected_plan(a_idx.cpu().numpy(), a_mask.cpu().numpy(), l_idx.cpu().numpy())
+    for label, packed in (("precompute", made), ("pack", pack_tree_mask(a_idx, a_mask, l_idx))):
+        got = packed.plan.cpu().numpy().view(np.uint32).reshape(nb, -1)
+        assert got.shape == want.shape, label
+        np.testing.assert_array_equal(got[care], want[care], err_msg=label)
+        assert (got[~care] < nb * block_m).all(), label      # spare keys name rows of the tree
+    # ids at or past the limit count as empty slots in a plan made by the packing entry point
+    limit = n // 2
+    want, care = expected_plan(a_idx.cpu().numpy(), a_mask.cpu().numpy(), l_idx.cpu().numpy(), key_limit=limit)
+    got = pack_tree_mask(a_idx, a_mask, l_idx, key_limit=limit).plan.cpu().numpy().view(np.uint32).reshape(nb, -1)
+    np.testing.assert_array_equal(got[care], want[care])
+    assert (got[~care] < limit).all()
+
+
 def test_lineage_from_parents_on_gpu():
     # (up to 16384 nodes the output rows are staged in LDS; larger trees are walked row by row)
     for seed, window, n in [(1, None, 777), (2, 8, 777), (3, 64, 777), (4, 2, 3000), (5, 40, 16384),
