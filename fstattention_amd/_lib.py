@@ -45,6 +45,7 @@ SIGNATURES = {
                                           c_void_p]),
     "fsta_dfs_order": (c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_void_p]),
+    "fsta_dfs_order_static": (c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]),
     "fsta_renumber_parents": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
     "fsta_medusa_tree": (c_int, [c_void_p, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p]),
     "fsta_merge_states": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,

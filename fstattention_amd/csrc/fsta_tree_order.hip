@@ -9,10 +9,37 @@
 //   off[i]   sum of size[s] over the siblings s visited before i (roots are siblings of each other)
 //   pre[i]   = sum over a in {i and its ancestors} of (off[a] + 1), minus 1
 //   perm[pre[i]] = i, rank[i] = pre[i]
+#include <mutex>
+
 #include "fsta_common.h"
 
 namespace fsta {
 namespace {
+
+// Scratch of fsta_dfs_order_static: subtree sizes and sibling offsets of one tree.  Every GPU the
+// library runs on holds its own copy of this array (128 KiB) at its own address until the process
+// ends; in host code the name below is only a handle for hipGetSymbolAddress, never an address.
+static __device__ __align__(256) int32_t scratch[2 * FSTA_DFS_ORDER_STATIC_MAX_NODES];
+
+constexpr int kMaxDevices = 64;
+int32_t* g_scratch_ptr[kMaxDevices] = {};   // device address of `scratch` on each device, once looked up
+std::mutex g_scratch_mutex;
+
+// Device address of the current device's copy of `scratch` (looked up on the first call per device).
+int scratch_on_current_device(int32_t** out) {
+    int dev = -1;
+    FSTA_HIP_OK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(FSTA_EUNSUPPORTED, "fsta_dfs_order_static: device %d", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        FSTA_HIP_OK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return fail(FSTA_EHIP, "fsta_dfs_order_static: no address for the scratch array");
+        g_scratch_ptr[dev] = static_cast<int32_t*>(ptr);
+    }
+    *out = g_scratch_ptr[dev];
+    return FSTA_OK;
+}
 
 constexpr int kOrderThreads = 256;
 constexpr int kSiblingTile = 256;    // candidate siblings staged in LDS per workgroup
@@ -249,16 +276,12 @@ extern "C" int fsta_renumber_parents(const int64_t* parent, const int64_t* rank,
     return FSTA_OK;
 }
 
-extern "C" int fsta_dfs_order(const int64_t* parent, int64_t n_nodes, int32_t light_first, int64_t* perm,
-                              int64_t* rank, int32_t* workspace, uint32_t* status, void* stream) {
-    if (n_nodes < 0) return fail(FSTA_EINVAL, "fsta_dfs_order: n_nodes=%lld", (long long)n_nodes);
-    if (n_nodes > FSTA_DFS_ORDER_MAX_NODES)
-        return fail(FSTA_EUNSUPPORTED, "fsta_dfs_order: n_nodes=%lld > %d (all-pairs sibling pass)",
-                    (long long)n_nodes, FSTA_DFS_ORDER_MAX_NODES);
-    if (n_nodes == 0) return FSTA_OK;
-    if (!parent || !perm || !rank || !workspace || !status)
-        return fail(FSTA_EINVAL, "fsta_dfs_order: null pointer");
-    hipStream_t s = static_cast<hipStream_t>(stream);
+namespace {
+
+// The launches of fsta_dfs_order; `workspace`: 2 * n_nodes int32 of device memory (only trees
+// too large for the single-workgroup kernel touch it).
+int dfs_order_launch(const int64_t* parent, int64_t n_nodes, int32_t light_first, int64_t* perm, int64_t* rank,
+                     int32_t* workspace, uint32_t* status, hipStream_t s) {
     if (n_nodes <= kSmallMaxNodes) {
         const size_t lds = (size_t)(6 * n_nodes + 3) * sizeof(int32_t);
         if (lds > 64 * 1024) {
@@ -280,6 +303,7 @@ extern "C" int fsta_dfs_order(const int64_t* parent, int64_t n_nodes, int32_t li
         if (rc == FSTA_OK) rc = allow_full_lds<&order_finish_kernel>();
         if (rc != FSTA_OK) return rc;
     }
+    // (size and off are set by a kernel: everything of an earlier call is overwritten)
     hipLaunchKernelGGL(order_init_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, n_nodes, size, off);
     hipLaunchKernelGGL(order_sizes_kernel, dim3(blocks), dim3(kOrderThreads), 2 * lds_parents, s, parent, n_nodes,
                        size, status);
@@ -289,4 +313,32 @@ extern "C" int fsta_dfs_order(const int64_t* parent, int64_t n_nodes, int32_t li
                        off, perm, rank, status);
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
+}
+
+}  // namespace
+
+extern "C" int fsta_dfs_order(const int64_t* parent, int64_t n_nodes, int32_t light_first, int64_t* perm,
+                              int64_t* rank, int32_t* workspace, uint32_t* status, void* stream) {
+    if (n_nodes < 0) return fail(FSTA_EINVAL, "fsta_dfs_order: n_nodes=%lld", (long long)n_nodes);
+    if (n_nodes > FSTA_DFS_ORDER_MAX_NODES)
+        return fail(FSTA_EUNSUPPORTED, "fsta_dfs_order: n_nodes=%lld > %d (all-pairs sibling pass)",
+                    (long long)n_nodes, FSTA_DFS_ORDER_MAX_NODES);
+    if (n_nodes == 0) return FSTA_OK;
+    if (!parent || !perm || !rank || !workspace || !status)
+        return fail(FSTA_EINVAL, "fsta_dfs_order: null pointer");
+    return dfs_order_launch(parent, n_nodes, light_first, perm, rank, workspace, status, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int fsta_dfs_order_static(const int64_t* parent, int64_t n_nodes, int32_t light_first, int64_t* perm,
+                                     int64_t* rank, uint32_t* status, void* stream) {
+    if (n_nodes < 0) return fail(FSTA_EINVAL, "fsta_dfs_order_static: n_nodes=%lld", (long long)n_nodes);
+    if (n_nodes > FSTA_DFS_ORDER_STATIC_MAX_NODES)
+        return fail(FSTA_EUNSUPPORTED, "fsta_dfs_order_static: n_nodes=%lld > %d (size of the library's own scratch array; "
+                    "fsta_dfs_order takes a workspace of the caller's)", (long long)n_nodes, FSTA_DFS_ORDER_STATIC_MAX_NODES);
+    if (n_nodes == 0) return FSTA_OK;
+    if (!parent || !perm || !rank || !status) return fail(FSTA_EINVAL, "fsta_dfs_order_static: null pointer");
+    int32_t* work = nullptr;
+    const int rc = scratch_on_current_device(&work);
+    if (rc != FSTA_OK) return rc;
+    return dfs_order_launch(parent, n_nodes, light_first, perm, rank, work, status, static_cast<hipStream_t>(stream));
 }

@@ -237,6 +237,22 @@ int fsta_dfs_order(const int64_t* parent, int64_t n_nodes, int32_t light_first, 
                    int64_t* rank, int32_t* workspace, uint32_t* status, void* stream);
 
 /*
+ * fsta_dfs_order without a workspace argument and without any allocation: the
+ * scratch (2 * n_nodes int32) is an array inside the library, one copy per GPU,
+ * held until the process ends (128 KiB).  No counterpart in the reference; for
+ * callers that cannot allocate device memory: code under HIP graph capture,
+ * serving loops and harnesses that forbid hipMalloc.  Same arguments, results
+ * and status bits as fsta_dfs_order; n_nodes <= FSTA_DFS_ORDER_STATIC_MAX_NODES,
+ * larger trees are refused with FSTA_EUNSUPPORTED.  All calls on one GPU share
+ * that GPU's array: calls that overlap on one GPU (two streams, two threads)
+ * race, queue them on one stream or order them with events.  The first call on
+ * a device looks the array's address up (no memory is allocated).
+ */
+#define FSTA_DFS_ORDER_STATIC_MAX_NODES 16384
+int fsta_dfs_order_static(const int64_t* parent, int64_t n_nodes, int32_t light_first, int64_t* perm,
+                          int64_t* rank, uint32_t* status, void* stream);
+
+/*
  * Joins two partial attention results of the same queries over disjoint key
  * sets: o = (o_a 2^lse_a + o_b 2^lse_b) / (2^lse_a + 2^lse_b) per row, lse_out
  * (may be NULL) = log2 of the denominator.  o_*: [rows, head_dim] of `dtype`,

@@ -1,0 +1,51 @@
+"""The entry point that allocates nothing (``fsta_dfs_order_static``) against ``fsta_dfs_order``.
+
+Through the C ABI: same parent arrays, results compared bit for bit, two calls in a row with the
+second tree smaller than the first (the library's scratch array keeps the first call's contents).
+Both trees are larger than what the single-workgroup kernel takes, so both calls use the scratch.
+"""
+import numpy as np
+import pytest
+import torch
+
+from fstattention_amd import _lib, trees
+
+pytestmark = pytest.mark.gpu
+
+
+def _order(lib, entry, parent, light_first, workspace):
+    n = parent.shape[0]
+    perm = torch.full((n,), -7, dtype=torch.int64, device="cuda")
+    rank = torch.full((n,), -7, dtype=torch.int64, device="cuda")
+    status = torch.zeros((1,), dtype=torch.int32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    if entry == "static":
+        rc = lib.fsta_dfs_order_static(parent.data_ptr(), n, light_first, perm.data_ptr(), rank.data_ptr(),
+                                       status.data_ptr(), stream)
+    else:
+        rc = lib.fsta_dfs_order(parent.data_ptr(), n, light_first, perm.data_ptr(), rank.data_ptr(),
+                                workspace.data_ptr(), status.data_ptr(), stream)
+    _lib.check(rc)
+    torch.cuda.synchronize()
+    return perm.cpu().numpy(), rank.cpu().numpy(), int(status.item())
+
+
+def test_static_scratch_entry_point_matches_the_workspace_one():
+    lib = _lib.load()
+    limit = 16384
+    for n, seed, window, light in ((12000, 5, 64, 1), (5000, 6, None, 0), (limit, 7, 8, 1), (4097, 8, 200, 0), (300, 9, 16, 1)):
+        host_parent = trees.random_recursive_parents(n, seed, window)
+        parent = torch.from_numpy(host_parent).cuda()
+        work = torch.full((2 * n,), 0x5A5A5A5A, dtype=torch.int32, device="cuda")
+        want = _order(lib, "workspace", parent, light, work)
+        got = _order(lib, "static", parent, light, None)
+        assert got[2] == 0 and want[2] == 0
+        np.testing.assert_array_equal(got[0], want[0], err_msg=f"perm, n={n}")
+        np.testing.assert_array_equal(got[1], want[1], err_msg=f"rank, n={n}")
+        np.testing.assert_array_equal(got[0], trees.dfs_order(host_parent, "light_first" if light else "index"))
+    # beyond the array's size: refused on the host, nothing launched; a malformed tree is flagged as by the other entry point
+    assert lib.fsta_dfs_order_static(parent.data_ptr(), limit + 1, 0, 8, 8, 8, None) == _lib.EUNSUPPORTED
+    assert b"scratch" in lib.fsta_last_error()
+    bad = torch.from_numpy(trees.random_recursive_parents(6000, 3, 32)).cuda()
+    bad[100] = 5000
+    assert _order(lib, "static", bad, 0, None)[2] & _lib.PRE_BAD_NODE_ID
