@@ -37,11 +37,27 @@ HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 INFINITY_CACHE_BYTES = 256 << 20
 
-# HBM bytes per launch of the headline kernel (256-node tree, cold buffers) from two
-# rocprofv3 --pmc runs, see profiles/attn_mfma16_kernel_cfg2_medusa256_hbm_traffic.txt:
-# FETCH_SIZE 3155.5 KiB x 2.0 (a plain 256 MiB copy reads 131084 KiB on this counter, i.e. the
-# counter sees half of the read traffic) + WRITE_SIZE 2080 KiB x 1.0 (the copy reads 262144).
-MEASURED_TRAFFIC_BYTES = int((3155.5 * 2 + 2080) * 1024)
+# HBM bytes per launch of the headline kernel come from a tracked rocprofv3 counter summary (two
+# --pmc runs, FETCH_SIZE and WRITE_SIZE, scaled by what the counters read for a plain copy); the
+# summary names the kernel it was taken from, and the figure is only reported for that kernel.
+TRAFFIC_PROFILE = os.path.join(REPO, "profiles", "attn_mfma16_kernel_cfg2_medusa256_hbm_traffic.txt")
+HEADLINE_MIN_STEPS = 400     # the headline is also timed over at least this many steps, whatever --steps says
+
+
+def measured_traffic(kernel_name):
+    """HBM bytes per launch from the tracked counter summary, if it was taken from `kernel_name`
+    (template arguments included), else None."""
+    import re
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return None
+    kernel = re.search(r"^kernel:\s*(.+)$", text, re.M)
+    traffic = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", text, re.M)
+    squeeze = lambda t: t.replace(" ", "")
+    if not kernel or not traffic or squeeze(kernel.group(1)) != squeeze(kernel_name.split(">")[0] + ">"):
+        return None
+    return int(traffic.group(1))
 
 
 def parse_args():
@@ -50,7 +66,10 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (headline: 2)")
-    ap.add_argument("--extra", action="store_true", help="also time configurations 3, 4 and 5")
+    ap.add_argument("--extra", action="store_true",
+                    help="also time the depth-first orderings, the front-end kernels, decoding steps and prefixes")
+    ap.add_argument("--quick", action="store_true",
+                    help="headline only: skip the other configurations and the reference's benchmark shapes")
     ap.add_argument("--regimes", action="store_true",
                     help="also time the warm-cache loop, plain stream launches, the Python entry point "
                          "and the GPU precompute")
@@ -71,14 +90,15 @@ class Workload:
     """Device-resident inputs of one configuration, in `sets` rotating copies."""
 
     def __init__(self, index, sets_bytes, dtype=None, heads=None, batch=None, order=None, prefix=0,
-                 key_splits=None):
+                 key_splits=None, device_rng=False):
         import torch
         from fstattention_amd import _lib, create_fst_attention_kernel_inputs, shift_for_prefix, trees
         from fstattention_amd.attention import _DTYPES, _packed_for
 
         self.torch = torch
-        self.cfg = cfg = trees.config(index, dtype)
-        self.cfg_index = index
+        # `index`: one of the five benchmark configurations, or a TreeConfig of the caller's
+        self.cfg = cfg = trees.config(index, dtype) if isinstance(index, int) else index
+        self.cfg_index = index if isinstance(index, int) else None
         if order is not None:
             # the same tree with its nodes (tokens) numbered depth-first (reference README.md:19-20)
             import dataclasses
@@ -89,7 +109,7 @@ class Workload:
         dev = torch.device("cuda", 0)
         self.z = batch or cfg.batch
         self.h = heads or cfg.heads
-        self.n, self.d, self.m = cfg.n_nodes, cfg.head_dim, cfg.block_m
+        self.n, self.d, self.m = cfg.n_nodes + cfg.pad_rows, cfg.head_dim, cfg.block_m
         self.dtype = cfg.dtype
         self.code = _DTYPES[cfg.dtype]
         self.esz = torch.tensor([], dtype=cfg.dtype).element_size()
@@ -98,7 +118,7 @@ class Workload:
         # kernel inputs: GPU precompute from the device-resident lineage
         lineage, level = trees.lineage_from_parents(cfg.parent)
         self.lineage, self.level = lineage.to(dev), level.to(dev)
-        self.max_anc = trees.required_max_ancestors(cfg.parent, self.m, 16)
+        self.max_anc = cfg.max_ancestors or trees.required_max_ancestors(cfg.parent, self.m, 16)
         self.a_idx, self.a_mask, self.l_idx = create_fst_attention_kernel_inputs(
             self.lineage, self.level, self.m, self.max_anc, mutate_lineage=False)
         # K/V laid out as [shared prefix | tree] (reference fstattention.py:209-212)
@@ -113,7 +133,7 @@ class Workload:
         self.kv_rows = rows + self.nb * prefix       # every block walks the whole prefix
         self.kv_bytes = self.z * self.h * 2 * self.d * self.esz * self.kv_rows
         depth = trees.levels_from_parents(cfg.parent)
-        self.pairs = int(depth.sum() + self.n) + self.n * prefix
+        self.pairs = int(depth.sum() + cfg.n_nodes) + cfg.n_nodes * prefix
         self.flops = 4 * self.d * self.z * self.h * self.pairs
 
         # HBM bytes a launch has to move at least once when nothing is cached from before:
@@ -121,7 +141,8 @@ class Workload:
         self.min_traffic_bytes = self.z * self.h * ((2 * self.n + 2 * self.nk) * self.d * self.esz + 4 * self.n)
         per_set = self.z * self.h * (2 * self.n + 2 * self.nk) * self.d * self.esz
         self.per_set_bytes = per_set
-        self.n_sets = max(2, min(256, -(-sets_bytes // per_set)))
+        # (one set that is larger than twice the Infinity Cache is cold by itself)
+        self.n_sets = max(1 if per_set >= 2 * INFINITY_CACHE_BYTES else 2, min(256, -(-sets_bytes // per_set)))
         shape = (self.z, self.h, self.n, self.d)
         kv_shape = (self.z, self.h, self.nk, self.d)
         # workspace for a prefix cut into runs of keys (none wanted: plain entry point)
@@ -134,7 +155,16 @@ class Workload:
         self.sets = []
         base = None
         for s in range(self.n_sets):
-            if s < 4 or base is None:
+            if device_rng and base is None:
+                # N(0,1) drawn on the device (seeded): the large configurations, timing only
+                gd = torch.Generator(device=dev).manual_seed(cfg.tensor_seed)
+                q, k, v = (torch.randn(sh, generator=gd, dtype=torch.float32, device=dev).to(cfg.dtype)
+                           if sh[0] * sh[1] * sh[2] * sh[3] <= 1 << 28 else
+                           torch.cat([torch.randn((1,) + sh[1:], generator=gd, dtype=torch.float32, device=dev).to(cfg.dtype)
+                                      for _ in range(sh[0])])
+                           for sh in (shape, kv_shape, kv_shape))
+                base = (q, k, v)
+            elif not device_rng and (s < 4 or base is None):
                 # CPU-seeded N(0,1), rounded to the storage type, then moved
                 q, k, v = (torch.randn(sh, generator=g, dtype=torch.float32).to(cfg.dtype).to(dev)
                            for sh in (shape, kv_shape, kv_shape))
@@ -424,6 +454,53 @@ def summarize(wl, steps, warmup, use_graph, regimes):
     return out
 
 
+def brief(w, steps, warmup, use_graph):
+    """Cold timing of one workload with the figures every configuration is reported with."""
+    ok, err, _ = w.cross_check()
+    wall, ev = time_steps(w, steps, warmup, rotate=True, use_graph=use_graph)
+    return {
+        "us_per_call_cold": round(wall * 1e6, 2), "kernel": w.lib.fsta_last_attention_kernel().decode(),
+        "kv_bytes_per_call": w.kv_bytes, "kv_gbps_cold": round(w.kv_bytes / ev / 1e9, 1),
+        "hbm_frac": round(w.kv_bytes / ev / 1e9 / HBM_PEAK_GBPS, 4),
+        "q_k_v_o_once_gbps": round(w.min_traffic_bytes / ev / 1e9, 1),
+        "effective_tflops": round(w.flops / ev / 1e12, 3),
+        "batch": w.z, "heads": w.h, "nodes": w.cfg.n_nodes, "block_m": w.m, "max_ancestors": w.max_anc,
+        "dtype": str(w.dtype).replace("torch.", ""), "buffer_sets": w.n_sets, "steps": steps,
+        "cross_check_ok": ok, "max_abs_diff_vs_scalar_kernel": err,
+    }
+
+
+def other_configurations(use_graph):
+    """The benchmark configurations beside the headline: 1 (float32, vector-ALU kernel), 3, 4 and 5
+    (configuration 5 on two buffer sets = 2 GiB, each larger than the Infinity Cache)."""
+    import torch
+    out = {}
+    for idx in (1, 3, 4, 5):
+        w = Workload(idx, sets_bytes=2 * INFINITY_CACHE_BYTES, device_rng=idx != 1)
+        out[w.cfg.name] = brief(w, 30 if idx == 5 else 100, 5, use_graph)
+        del w
+        torch.cuda.empty_cache()
+    return out
+
+
+def reference_benchmark(use_graph):
+    """The workload the reference's own benchmark is quoted on (fstattention.py:240-296): batch 4, 48 heads,
+    head dim 64, float16, create_tree(DEPTH_MAPPING[N]) for N = 2^10 .. 2^16, blocks of 128 rows, 64
+    ancestor slots; the reference reports milliseconds per call of the attention operator."""
+    import torch
+    from fstattention_amd import trees
+    out = {}
+    for k in range(10, 17):
+        w = Workload(trees.reference_benchmark_config(2 ** k), sets_bytes=2 * INFINITY_CACHE_BYTES, device_rng=True)
+        b = brief(w, 20 if k >= 15 else 50, 3, use_graph)
+        out[f"n_ctx_{2 ** k}"] = {key: b[key] for key in ("us_per_call_cold", "kv_bytes_per_call", "kv_gbps_cold", "hbm_frac",
+                                                         "q_k_v_o_once_gbps", "buffer_sets", "cross_check_ok", "kernel")}
+        out[f"n_ctx_{2 ** k}"]["ms_per_call"] = round(b["us_per_call_cold"] / 1e3, 4)
+        del w
+        torch.cuda.empty_cache()
+    return out
+
+
 def copy_calibration(mib):
     """10 plain device copies of `mib` MiB: what FETCH_SIZE / WRITE_SIZE read for known traffic."""
     import torch
@@ -468,12 +545,19 @@ def main():
         sys.exit(1)
 
     t = summarize(wl, args.steps, args.warmup, use_graph, args.regimes)
+    kernel_name = wl.lib.fsta_last_attention_kernel().decode()
     step_s = t["cold_us"] * 1e-6
-    kernel_s = t["cold_event_us"] * 1e-6
+    # the dominant kernel's average launch duration: HIP events on the launch stream around a graph of
+    # at least HEADLINE_MIN_STEPS launches (a 20-step region is 0.1 ms, too short to trust on its own)
+    long_steps = max(args.steps, HEADLINE_MIN_STEPS)
+    long_wall, long_ev = (t["cold_us"] * 1e-6, t["cold_event_us"] * 1e-6) if long_steps == args.steps else \
+        time_steps(wl, long_steps, args.warmup, rotate=True, use_graph=use_graph)
+    kernel_s = long_ev
     achieved = wl.kv_bytes / kernel_s / 1e9
+    headline = args.config == 2 and not args.prefix
     result = {
         "metric": "K/V GB/s loaded (us/call in us_per_call), 256-node Medusa tree H32 D128 bf16"
-                  if args.config == 2 and not args.prefix else
+                  if headline else
                   f"K/V GB/s loaded, {wl.cfg.name}" + (f" behind {args.prefix} prefix keys" if args.prefix else ""),
         "value": round(wl.kv_bytes / step_s / 1e9, 2),
         "unit": "GB/s",
@@ -495,19 +579,20 @@ def main():
                             f", {wl.n_sets} rotating q/k/v/o sets ({wl.n_sets * wl.per_set_bytes >> 20} MiB)",
         },
         "effective_tflops": round(wl.flops / step_s / 1e12, 4),
+        "same_loop_over_more_steps": {"steps": long_steps, "us_per_call": round(long_wall * 1e6, 3),
+                                      "value": round(wl.kv_bytes / long_wall / 1e9, 2)},
         "cross_check": {"max_abs_diff_vs_scalar_kernel": max_err, "tol": tol, "ok": ok},
         "roofline": {
             "bound": "hbm",
-            "kernel": ("attn_generic_kernel" if wl.dtype == torch.float32 else
-                       "attn_mfma16_kernel<bf16, D=128, 32-row halves of the 64-row blocks, split P, wave pairs by head-dim halves>"
-                       if args.config == 2 and wl.dtype == torch.bfloat16 and not args.prefix else "attn_mfma16_kernel"),
+            "kernel": kernel_name,
             "achieved": round(achieved, 2),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 5),
-            "traffic": MEASURED_TRAFFIC_BYTES if args.config == 2 and not args.prefix else None,
+            "traffic": measured_traffic(kernel_name) if headline and wl.dtype == torch.bfloat16 else None,
             "algorithmic_bytes_per_launch": wl.kv_bytes,
             "avg_launch_us": round(kernel_s * 1e6, 3),
+            "launches_timed": long_steps,
             "mfma_frac_of_bf16_peak": round(wl.flops / kernel_s / 1e12 / MFMA_BF16_PEAK_TFLOPS, 6),
         },
     }
@@ -526,12 +611,15 @@ def main():
         if not result["parity"]["ok"]:
             print(f"bench.py: parity against the CPU oracle failed: {result['parity']}", file=sys.stderr)
             sys.exit(1)
+    if not args.quick and not args.prefix:
+        result["configs"] = other_configurations(use_graph)
+        result["reference_benchmark"] = reference_benchmark(use_graph)
     if args.extra:
         extra = {}
         for idx in (3, 4, 5):
             # configuration 5 is a 32-layer decoding step: one tree, 32 layers with their own q/k/v/o
             # (34 GB resident), so its buffer rotation is the layer loop itself
-            w = Workload(idx, sets_bytes=(32 << 30) if idx == 5 else 2 * INFINITY_CACHE_BYTES)
+            w = Workload(idx, sets_bytes=(32 << 30) if idx == 5 else 2 * INFINITY_CACHE_BYTES, device_rng=True)
             ok_i, err_i, _ = w.cross_check()
             steps = max(20, min(args.steps, 100 if idx == 5 else args.steps))
             ti = summarize(w, steps, min(args.warmup, 10), use_graph, True)

@@ -25,6 +25,7 @@ ABI_VERSION = 2
 SIGNATURES = {
     "fsta_abi_version": (c_int, []),
     "fsta_last_error": (c_char_p, []),
+    "fsta_last_attention_kernel": (c_char_p, []),
     "fsta_mask_words": (c_int32, [c_int32]),
     "fsta_block_plan_bytes": (c_size_t, [c_int32, c_int32, c_int32]),
     "fsta_precompute": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int32, c_int32,

@@ -9,6 +9,8 @@
 // mask), then the block's own rows through the diagonal "leaf" path
 // (fstattention.py:86-91), then the dense shared prefix (fstattention.py:113-136).
 // All three feed one online softmax in float32 (base 2, fstattention.py:55-59).
+#include <type_traits>
+
 #include "fsta_common.h"
 
 namespace fsta {
@@ -285,6 +287,8 @@ int launch_one(const AttnParams& p, hipStream_t stream) {
     dim3 grid(p.nb, p.heads_total);
     hipLaunchKernelGGL((attn_generic_kernel<T, D, M>), grid, dim3(kThreads), lds, stream, p);
     FSTA_HIP_OK(hipGetLastError());
+    note_launch({"attn_generic_kernel", sizeof(T) == 4 ? "float" : (std::is_same<T, __half>::value ? "__half" : "__hip_bfloat16"),
+                 {D, M, 0, 0, 0}, 2, 0u, 0, 0});
     return FSTA_OK;
 }
 

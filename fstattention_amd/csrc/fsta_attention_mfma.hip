@@ -500,6 +500,7 @@ int launch_one(const AttnParams& p, hipStream_t stream) {
     hipLaunchKernelGGL((attn_mfma_kernel<BF16, D, M, SPLIT>), dim3(grid), dim3(M * 2 * key_split_for(M)), lds,
                        stream, p, stages);
     FSTA_HIP_OK(hipGetLastError());
+    note_launch({"attn_mfma_kernel", BF16 ? "true" : "false", {D, M, SPLIT ? 1 : 0, 0, 0}, 3, 0x4u, 0, 0});
     return FSTA_OK;
 }
 

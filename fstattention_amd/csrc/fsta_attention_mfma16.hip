@@ -763,6 +763,8 @@ int launch_ks(const AttnParams& p, int sub_shift, hipStream_t stream) {
                            stream, p, stages, early, shift_arg);
     }
     FSTA_HIP_OK(hipGetLastError());
+    note_launch({"attn_mfma16_kernel", BF16 ? "true" : "false", {D, M, SPLIT ? 1 : 0, KS, p.key_splits > 1 ? 1 : 0}, 5,
+                 0x14u, sub_shift, early});
     return FSTA_OK;
 }
 

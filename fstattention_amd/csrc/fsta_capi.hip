@@ -16,9 +16,27 @@ int fail(int code, const char* fmt, ...) {
     return code;
 }
 
+static thread_local LaunchNote g_note = {nullptr, "", {0, 0, 0, 0, 0}, 0, 0u, 0, 0};
+static thread_local char g_note_text[192] = "";
+
+void note_launch(const LaunchNote& note) { g_note = note; }
+
 }  // namespace fsta
 
 using namespace fsta;
+
+extern "C" const char* fsta_last_attention_kernel(void) {
+    if (!g_note.kernel) return "";
+    int len = snprintf(g_note_text, sizeof(g_note_text), "%s<%s", g_note.kernel, g_note.first);
+    for (int i = 0; i < g_note.n_args && len < (int)sizeof(g_note_text); ++i)
+        len += (g_note.bool_args >> i) & 1u
+                   ? snprintf(g_note_text + len, sizeof(g_note_text) - len, ", %s", g_note.args[i] ? "true" : "false")
+                   : snprintf(g_note_text + len, sizeof(g_note_text) - len, ", %d", g_note.args[i]);
+    if (len < (int)sizeof(g_note_text))
+        snprintf(g_note_text + len, sizeof(g_note_text) - len, ">%s%s", g_note.half_blocks ? " half-blocks" : "",
+                 g_note.early_start ? " early-start" : "");
+    return g_note_text;
+}
 
 extern "C" int fsta_abi_version(void) { return FSTA_ABI_VERSION; }
 

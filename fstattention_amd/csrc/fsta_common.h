@@ -90,6 +90,18 @@ int allow_full_lds() {
     return FSTA_OK;
 }
 
+// Which attention kernel the calling thread launched last (fsta_last_attention_kernel): the kernel's
+// name and up to six template arguments, kept as numbers and turned into text only when asked for.
+struct LaunchNote {
+    const char* kernel;   // string literal
+    const char* first;    // first template argument as text, e.g. "true" or "float"
+    int args[5];
+    int n_args;
+    unsigned bool_args;   // bit i: args[i] is a bool template argument
+    int half_blocks, early_start;   // launch options of the narrow matrix-core kernel
+};
+void note_launch(const LaunchNote& note);
+
 // launchers, one per translation unit
 int launch_attention_generic(const AttnParams& p, int dtype, int head_dim, hipStream_t stream);
 int launch_attention_mfma(const AttnParams& p, int dtype, int head_dim, bool fast_pv,

@@ -224,6 +224,8 @@ class TreeConfig:
     tree_seed: int
     tensor_seed: int
     layers: int = 1
+    pad_rows: int = 0          # q/k/v rows past the tree (the reference's tensors hold N_CTX = n_nodes + 4 rows)
+    max_ancestors: int = 0     # 0: derived from the tree
 
     @property
     def n_nodes(self) -> int:
@@ -339,6 +341,16 @@ def config(index: int, dtype: torch.dtype | None = None) -> TreeConfig:
         return TreeConfig("cfg5_batched2048", random_recursive_parents(2048, 1005, window=64), 128,
                           8, 64, 128, dtype or torch.bfloat16, 1005, 2005, layers=32)
     raise ValueError(f"no such config: {index}")
+
+
+def reference_benchmark_config(n_ctx: int) -> TreeConfig:
+    """The workload of the reference's own benchmark (``fstattention.py:240-296``): batch 4, 48 heads,
+    head dim 64, float16, ``create_tree(DEPTH_MAPPING[n_ctx])`` (``n_ctx - 4`` nodes in tensors of
+    ``n_ctx`` rows), query blocks of 128 rows, 64 ancestor slots."""
+    lineage, level = create_tree(DEPTH_MAPPING[n_ctx])
+    parent = parents_from_lineage(lineage.numpy(), level.numpy())
+    return TreeConfig(f"reference_benchmark_n{n_ctx}", parent, 128, 4, 48, 64, torch.float16, 0, 3000 + n_ctx,
+                      pad_rows=n_ctx - parent.shape[0], max_ancestors=MAX_ANCESTOR_MAPPING[n_ctx])
 
 
 def make_qkv(cfg: TreeConfig, layer: int = 0, device="cpu", prefix: int = 0):

@@ -65,6 +65,11 @@ int fsta_abi_version(void);
 /* Message of the last failing call made by this thread ("" if none). */
 const char* fsta_last_error(void);
 
+/* Which attention kernel the last fsta_attention_fwd* call of this thread launched, as
+ * "name<template arguments>" in the spelling profilers show (e.g. rocprofv3's kernel trace),
+ * followed by launch options; "" before the first launch.  For benchmarks and profiles. */
+const char* fsta_last_attention_kernel(void);
+
 /* Number of 32-bit words per (block, query row) in the packed tree mask. */
 int32_t fsta_mask_words(int32_t max_ancestors);
 
