@@ -90,7 +90,7 @@ class Workload:
     """Device-resident inputs of one configuration, in `sets` rotating copies."""
 
     def __init__(self, index, sets_bytes, dtype=None, heads=None, batch=None, order=None, prefix=0,
-                 key_splits=None, device_rng=False):
+                 key_splits=None, device_rng=False, kv8=False):
         import torch
         from fstattention_amd import _lib, create_fst_attention_kernel_inputs, shift_for_prefix, trees
         from fstattention_amd.attention import _DTYPES, _packed_for
@@ -131,15 +131,18 @@ class Workload:
         self.nb = self.a_idx.shape[0]
         rows = int((self.a_idx >= 0).sum().item() + (self.l_idx >= 0).sum().item())
         self.kv_rows = rows + self.nb * prefix       # every block walks the whole prefix
-        self.kv_bytes = self.z * self.h * 2 * self.d * self.esz * self.kv_rows
+        # 8-bit K/V storage: K and V rows are float8_e4m3fn with a scale per (batch, head) slice
+        self.kv8 = kv8
+        self.kv_esz = 1 if kv8 else self.esz
+        self.kv_bytes = self.z * self.h * 2 * self.d * self.kv_esz * self.kv_rows
         depth = trees.levels_from_parents(cfg.parent)
         self.pairs = int(depth.sum() + cfg.n_nodes) + cfg.n_nodes * prefix
         self.flops = 4 * self.d * self.z * self.h * self.pairs
 
         # HBM bytes a launch has to move at least once when nothing is cached from before:
         # every K and V row, Q, O and the log-sum-exp (rows shared by blocks come from L2)
-        self.min_traffic_bytes = self.z * self.h * ((2 * self.n + 2 * self.nk) * self.d * self.esz + 4 * self.n)
-        per_set = self.z * self.h * (2 * self.n + 2 * self.nk) * self.d * self.esz
+        self.min_traffic_bytes = self.z * self.h * ((2 * self.n * self.esz + 2 * self.nk * self.kv_esz) * self.d + 4 * self.n)
+        per_set = self.z * self.h * (2 * self.n * self.esz + 2 * self.nk * self.kv_esz) * self.d
         self.per_set_bytes = per_set
         # (one set that is larger than twice the Infinity Cache is cold by itself)
         self.n_sets = max(1 if per_set >= 2 * INFINITY_CACHE_BYTES else 2, min(256, -(-sets_bytes // per_set)))
@@ -174,6 +177,9 @@ class Workload:
                 # memory, same distribution) so that building them stays cheap
                 q, k, v = (torch.roll(t, shifts=s, dims=2).contiguous() for t in base)
             o = torch.empty(shape, dtype=cfg.dtype, device=dev)
+            if kv8:
+                from fstattention_amd import quantize_kv_fp8
+                k, v, self.k_scale, self.v_scale = quantize_kv_fp8(k, v)     # (every set is a roll of the first: same scales)
             self.sets.append((q, k, v, o))
         self.lse = torch.empty((self.z * self.h, self.n), dtype=torch.float32, device=dev)
 
@@ -181,6 +187,12 @@ class Workload:
         """One step: a single call through the C ABI on torch's current stream."""
         torch = self.torch
         q, k, v, o = self.sets[s % self.n_sets]
+        if self.kv8:
+            self._check(self.lib.fsta_attention_fwd_kv8(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), self.k_scale.data_ptr(), self.v_scale.data_ptr(), o.data_ptr(),
+                self.lse.data_ptr(), self.plan_ptr, self.packed.key_shift, self.z, self.h, self.n, self.nk, self.d,
+                self.code, self.code, self.m, self.max_anc, self.nb, self.scale, torch.cuda.current_stream().cuda_stream))
+            return
         if self.work is not None:
             self._check(self.lib.fsta_attention_fwd_ws(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), self.lse.data_ptr(),
@@ -205,8 +217,11 @@ class Workload:
         q, k, v, _ = self.sets[0]
         hh = min(heads, self.h)
         self._sample = tuple(t[:1, :hh].contiguous() for t in (q, k, v))
+        self._sample_scales = {}
+        if self.kv8:
+            self._sample_scales = {"k_scale": self.k_scale[:hh].contiguous(), "v_scale": self.v_scale[:hh].contiguous()}
         return fst_attention(*self._sample, self.a_idx, self.a_mask, self.l_idx, self.scale,
-                             BLOCK_M=self.m, MAX_ANCESTORS=self.max_anc, out_dtype=torch.float32)
+                             BLOCK_M=self.m, MAX_ANCESTORS=self.max_anc, out_dtype=torch.float32, **self._sample_scales)
 
     def cross_check(self, heads=2):
         """Default kernel vs the library's scalar kernel (an independent second implementation)
@@ -216,7 +231,12 @@ class Workload:
         torch = self.torch
         from fstattention_amd import fst_attention
         o = self.run_default(heads)
-        ref = fst_attention(*self._sample, self.a_idx, self.a_mask, self.l_idx, self.scale,
+        sample = self._sample
+        if self.kv8:      # the scalar kernel in float32 on the widened rows (a 16-bit copy of them would be rounded again)
+            qs, k8, v8 = sample
+            widen = lambda t, sc: t.float() * sc.view(1, -1, 1, 1)
+            sample = (qs.float(), widen(k8, self._sample_scales["k_scale"]), widen(v8, self._sample_scales["v_scale"]))
+        ref = fst_attention(*sample, self.a_idx, self.a_mask, self.l_idx, self.scale,
                             BLOCK_M=self.m, MAX_ANCESTORS=self.max_anc, out_dtype=torch.float32, generic=True)
         tol = 1e-5 if self.dtype == torch.float32 else 2e-3
         err = (o.double() - ref.double()).abs()
@@ -501,6 +521,31 @@ def reference_benchmark(use_graph):
     return out
 
 
+def fp8_kv_storage(use_graph):
+    """16-bit against 8-bit K/V storage where the 16-bit kernel already runs near the rate of a plain copy:
+    configuration 4, configuration 5 with its tokens in depth-first order, one of the reference's benchmark shapes."""
+    import torch
+    from fstattention_amd import trees
+    cases = (("cfg4_wide4096", lambda kv8: Workload(4, 2 * INFINITY_CACHE_BYTES, device_rng=True, kv8=kv8), 100),
+             ("cfg5_batched2048_depth_first", lambda kv8: Workload(5, 2 * INFINITY_CACHE_BYTES, device_rng=True,
+                                                                   order="light_first", kv8=kv8), 30),
+             ("reference_benchmark_n16384", lambda kv8: Workload(trees.reference_benchmark_config(16384),
+                                                                 2 * INFINITY_CACHE_BYTES, device_rng=True, kv8=kv8), 30))
+    out = {}
+    for name, make, steps in cases:
+        entry = {}
+        for label, kv8 in (("k_v_16bit", False), ("k_v_fp8_e4m3", True)):
+            w = make(kv8)
+            b = brief(w, steps, 3, use_graph)
+            entry[label] = {key: b[key] for key in ("us_per_call_cold", "kv_bytes_per_call", "kv_gbps_cold", "hbm_frac",
+                                                    "q_k_v_o_once_gbps", "cross_check_ok", "kernel")}
+            entry[label]["q_k_v_o_once_bytes"] = w.min_traffic_bytes
+            del w
+            torch.cuda.empty_cache()
+        out[name] = entry
+    return out
+
+
 def copy_calibration(mib):
     """10 plain device copies of `mib` MiB: what FETCH_SIZE / WRITE_SIZE read for known traffic."""
     import torch
@@ -614,6 +659,7 @@ def main():
     if not args.quick and not args.prefix:
         result["configs"] = other_configurations(use_graph)
         result["reference_benchmark"] = reference_benchmark(use_graph)
+        result["fp8_kv_storage"] = fp8_kv_storage(use_graph)
     if args.extra:
         extra = {}
         for idx in (3, 4, 5):

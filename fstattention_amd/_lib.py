@@ -42,6 +42,9 @@ SIGNATURES = {
                                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32,
                                       c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
                                       c_int32, c_int32, c_int32, c_float, c_uint32, c_void_p, c_size_t, c_void_p]),
+    "fsta_attention_fwd_kv8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                       c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
+                                       c_int32, c_int32, c_float, c_void_p]),
     "fsta_lineage_from_parents": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
                                           c_void_p]),
     "fsta_dfs_order": (c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,

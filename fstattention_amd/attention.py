@@ -148,10 +148,30 @@ def _packed_for(ancestor_idx: torch.Tensor, ancestor_mask, leaf_idx: torch.Tenso
     return packed
 
 
+_FP8 = torch.float8_e4m3fn
+_FP8_MAX = 448.0
+
+
+def quantize_kv_fp8(k: torch.Tensor, v: torch.Tensor):
+    """``k, v [Z,H,Nk,D]`` -> ``(k8, v8, k_scale, v_scale)`` for ``fst_attention``'s 8-bit K/V storage:
+    ``float8_e4m3fn`` tensors and one float32 scale per (batch, head) slice (``[Z*H]``) chosen so that
+    the slice's largest magnitude maps to the format's largest value (448).  ``k8 * k_scale`` is the K
+    the kernel computes with.  Plain tensor operations; a model would write its KV cache this way."""
+    def one(t):
+        amax = t.float().abs().amax(dim=(2, 3))
+        scale = torch.where(amax > 0, amax / _FP8_MAX, torch.ones_like(amax))
+        t8 = (t.float() / scale[:, :, None, None]).to(_FP8)
+        return t8.contiguous(), scale.reshape(-1).contiguous()
+    k8, k_scale = one(k)
+    v8, v_scale = one(v)
+    return k8, v8, k_scale, v_scale
+
+
 def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
                   BLOCK_M=128, MAX_ANCESTORS=64, *, out_dtype: Optional[torch.dtype] = None,
                   return_lse: bool = False, fast_pv: bool = False, generic: bool = False,
-                  wide_waves: bool = False, key_splits: Optional[int] = None, share_tiles: bool = False):
+                  wide_waves: bool = False, key_splits: Optional[int] = None, share_tiles: bool = False,
+                  k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None):
     """Fused sparse tree attention forward (reference ``fstattention.py:153-181``).
 
     ``q [Z,H,Nq,D]``, ``k,v [Z,H,Nk,D]`` (``Nk - Nq`` leading rows are a dense
@@ -170,7 +190,11 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
     results live in a temporary workspace and are joined by a second kernel);
     ``key_splits`` forces the number of runs (``1``: never split); ``share_tiles`` is a tuning
     switch (wave pairs of a row group take alternate key tiles even where the library would let
-    them share the head dimension).  Inputs the reference silently
+    them share the head dimension).  ``k`` and ``v`` may be ``torch.float8_e4m3fn`` (8-bit K/V
+    storage, half the K/V bytes; ``q`` stays float16/bfloat16) with ``k_scale`` / ``v_scale`` float32
+    ``[Z*H]`` per-slice scales (``quantize_kv_fp8`` makes all four): the result is that of the 16-bit
+    call on ``k * k_scale`` and ``v * v_scale``; block sizes 32/64/128 and head dims 64/128 only, and
+    none of the kernel-selection switches apply.  Inputs the reference silently
     mis-handles raise ``ValueError`` here (non-contiguous tensors, index
     tensors whose shapes do not match ``BLOCK_M`` / ``MAX_ANCESTORS``).
     """
@@ -184,9 +208,18 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
         raise ValueError("fst_attention runs on the GPU only (no CPU fallback); move q/k/v to 'cuda'")
     if not (q.device == k.device == v.device == ancestor_idx.device == leaf_idx.device):
         raise ValueError("all tensors must live on the same device")
-    if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
+    kv8 = k.dtype == _FP8
+    if kv8:
+        if v.dtype != _FP8 or q.dtype not in (torch.float16, torch.bfloat16):
+            raise ValueError(f"8-bit K/V: k and v must both be float8_e4m3fn and q float16/bfloat16, got "
+                             f"{q.dtype}, {k.dtype}, {v.dtype}")
+        if fast_pv or generic or wide_waves or key_splits or share_tiles:
+            raise ValueError("8-bit K/V has one kernel: fast_pv, generic, wide_waves, key_splits and share_tiles do not apply")
+    elif q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
         raise ValueError(f"q/k/v must share one dtype of float32/float16/bfloat16, got "
                          f"{q.dtype}, {k.dtype}, {v.dtype}")
+    if (k_scale is not None or v_scale is not None) and not kv8:
+        raise ValueError("k_scale / v_scale belong to 8-bit K/V (float8_e4m3fn k and v)")
     if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
         raise ValueError("q, k, v must be contiguous")
     Z, H, Nq, D = q.shape
@@ -225,6 +258,21 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
     flags = (_lib.FLAG_FAST_PV if fast_pv else 0) | (_lib.FLAG_GENERIC if generic else 0) | \
         (_lib.FLAG_WIDE_WAVES if wide_waves else 0) | (_lib.flag_key_splits(key_splits) if key_splits else 0) | \
         (_lib.FLAG_SHARE_TILES if share_tiles else 0)
+    if kv8:
+        for name, scale in (("k_scale", k_scale), ("v_scale", v_scale)):
+            if scale is not None and (scale.dtype != torch.float32 or scale.numel() != Z * H or
+                                      scale.device != q.device or not scale.is_contiguous()):
+                raise ValueError(f"{name} must be a contiguous float32 tensor of {Z * H} entries on {q.device}")
+        if plan_ptr is None:
+            raise ValueError(f"8-bit K/V needs BLOCK_M of 32, 64 or 128 (got {BLOCK_M})")
+        with _on_device(q.device):
+            _lib.check(lib.fsta_attention_fwd_kv8(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), k_scale.data_ptr() if k_scale is not None else None,
+                v_scale.data_ptr() if v_scale is not None else None, o.data_ptr(),
+                lse.data_ptr() if return_lse else None, plan_ptr, packed.key_shift, Z, H, Nq, Nk, D,
+                _DTYPES[q.dtype], _DTYPES[out_dtype], BLOCK_M, MAX_ANCESTORS, nb, float(sm_scale),
+                _stream_ptr(q.device)))
+        return (o, lse) if return_lse else o
     # a shared prefix may be worth cutting into key runs: the library says how much workspace that takes
     work, work_bytes = None, 0
     if Nk > Nq:

@@ -72,7 +72,12 @@ __device__ __forceinline__ void flush_rows(const unsigned char* stage, int strid
 // of a launch with one or two ancestor tiles per block; the duplicated S and softmax work makes
 // it the wrong choice for long tile lists.
 // RUNS = the launch cuts the shared prefix into runs of keys (AttnParams::key_splits > 1).
-template <bool BF16, int D, int M, bool SPLIT, int KS, bool RUNS>
+// KV8 = K and V are stored as 8-bit floats (OCP e4m3) with one scale per (batch, head) slice each:
+// rows are gathered as they are (half the bytes) into a staging ring; the workgroup widens every
+// tile once into one of two 16-bit tiles in LDS (exact: e4m3 is a subset of both 16-bit types),
+// one step ahead of its use, and the products run on those as they do for 16-bit K/V.  Widening a
+// tile once per workgroup costs an eighth of widening the fragments in every wave.
+template <bool BF16, int D, int M, bool SPLIT, int KS, bool RUNS, bool KV8 = false>
 __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_kernel(AttnParams p, int stages, int early_leaf, int sub_shift) {
     using MM = Mma<BF16>;
     using T = typename MM::elem;
@@ -84,10 +89,14 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     constexpr int kSplit = kDShare ? 1 : KS;      // tiles per step, dealt to the waves of a row group
     constexpr int kShares = kDShare ? -KS : KS;   // waves per row group
     static_assert(!kDShare || (KS == -2 && D >= 64), "head-dimension halves need two accumulator tiles each");
-    constexpr int kLeafGroup = leaf_group16_for(M);
+    static_assert(!KV8 || (KS == 1 && !RUNS), "8-bit K/V: one wave per row group, no key runs");
+    constexpr int kLeafGroup = KV8 ? 1 : leaf_group16_for(M);
     constexpr int kWaves = kQGroups * kShares;
-    constexpr int kCpr = D / 8;                   // 16-byte chunks per row
-    constexpr int kRowsPerDma = 64 / kCpr;        // rows one wave-wide 1 KiB transfer covers
+    constexpr int kThreads = kWaves * 64;
+    constexpr int kCpr = D / 8;                   // 16-byte chunks per 16-bit row (Q rows, tiles in LDS)
+    constexpr int kKvRowBytes = KV8 ? D : 2 * D;  // a K/V row in memory
+    constexpr int kKvCpr = kKvRowBytes / 16;      // 16-byte chunks per gathered row
+    constexpr int kRowsPerDma = 64 / kKvCpr;      // rows one wave-wide 1 KiB transfer covers
     constexpr int kDmaPerTile = 2 * kTileN / kRowsPerDma;   // K and V transfers of one tile
     constexpr int kDmaWaves = kDmaPerTile < kWaves ? kDmaPerTile : kWaves;   // waves that gather
     constexpr int kDmaPerWave = kDmaPerTile / kDmaWaves;
@@ -103,12 +112,17 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     constexpr float kTrustedSum = BF16 ? 16777216.f : 32768.f;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    T* ring = reinterpret_cast<T*>(smem);                 // [stages][K tile | V tile]
+    // 16-bit K/V: ring [stages][K tile | V tile].  8-bit K/V: two widened tiles [2][K tile | V tile],
+    // then the staging ring [stages][K rows | V rows] of bytes.
+    T* ring = reinterpret_cast<T*>(smem);
+    constexpr int kStageBytes = 2 * kTileN * D;           // one staged 8-bit tile
+    unsigned char* stage8 = smem + 2 * 2 * kTileElems * 2;
+    const int ring_bytes = KV8 ? 2 * 2 * kTileElems * 2 + stages * kStageBytes : stages * 2 * kTileElems * 2;
     // this workgroup's part of the block plan: header | ancestor keys | per 32 rows: leaf keys, mask words
     const int anc_cap = anc_tile_capacity(p.max_anc);
     const int common_words = kPlanHeaderWords + anc_cap * kTileN;
     const int group_words = kTileN * (1 + anc_cap);
-    uint32_t* plan_s = reinterpret_cast<uint32_t*>(ring + stages * 2 * kTileElems);
+    uint32_t* plan_s = reinterpret_cast<uint32_t*>(smem + ring_bytes);
     uint32_t* group_s = plan_s + common_words;            // [kLeafTiles][group_words]
 
     // All kernel arguments are fetched by ONE batch of scalar loads.  Left to itself the compiler
@@ -165,8 +179,11 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     const int row_in_block = qgroup * 16 + ql;
 
     const T* qb = static_cast<const T*>(p.q) + (size_t)hz * p.nq * D;
-    const T* kb = static_cast<const T*>(p.k) + (size_t)hz * p.nk * D;
-    const T* vb = static_cast<const T*>(p.v) + (size_t)hz * p.nk * D;
+    const unsigned char* kb = static_cast<const unsigned char*>(p.k) + (size_t)hz * p.nk * kKvRowBytes;
+    const unsigned char* vb = static_cast<const unsigned char*>(p.v) + (size_t)hz * p.nk * kKvRowBytes;
+    // scale under the exp2: softmax scale, log2(e) and, for 8-bit K, the slice's K scale
+    float sc = p.scale_log2e;
+    if (KV8 && p.k_scale) sc *= p.k_scale[hz];
 
     // ---- start-up: every request that needs no metadata goes out together with the metadata ----
     // Loads and transfers retire in issue order.  The block plan goes first (the ancestor requests
@@ -200,19 +217,24 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     // Q rows of this wave: whole rows straight into LDS, K-tile swizzle, parked in the last ring
     // slots until the fragments have been read (before the first barrier).  Rows past the end of
     // a ragged last block are read as the last row and never stored.
-    const int dma_row = lane / kCpr, dma_slot = lane % kCpr;
-    constexpr int kQDma = 16 / kRowsPerDma;
+    const int q_row = lane / kCpr, q_slot = lane % kCpr;           // Q rows are 16-bit
+    const int dma_row = lane / kKvCpr, dma_slot = lane % kKvCpr;   // K/V rows as stored
+    constexpr int kQRowsPerDma = 64 / kCpr;
+    constexpr int kQDma = 16 / kQRowsPerDma;
     static_assert(kQDma >= 1, "a transfer covers at most the wave's 16 rows");
     // (a small grid has LDS to spare: Q then gets an area of its own behind the plan, the
     // whole ring is free from the start and the fragments are read after the ancestor tiles have
     // been requested instead of in front of the first barrier)
+    // (8-bit K/V: Q waits in the widened tiles, which are first written behind the first barrier)
     T* qstage = early_leaf ? reinterpret_cast<T*>(group_s + kLeafTiles * group_words) + wave * 16 * D
+                : KV8      ? ring + wave * 16 * D
                            : ring + (size_t)stages * 2 * kTileElems - (kWaves - wave) * 16 * D;
+    static_assert(!KV8 || kWaves * 16 <= 4 * kTileN, "Q must fit into the two widened tiles");
 #pragma unroll
     for (int i = 0; i < kQDma; ++i) {
-        const int r = i * kRowsPerDma + dma_row;
+        const int r = i * kQRowsPerDma + q_row;
         const int grow = min(row_base + qgroup * 16 + r, p.nq - 1);
-        const uint32_t off = (uint32_t)grow * (uint32_t)(D * sizeof(T)) + (uint32_t)k_chunk<D>(r, dma_slot) * 16u;
+        const uint32_t off = (uint32_t)grow * (uint32_t)(D * sizeof(T)) + (uint32_t)k_chunk<D>(r, q_slot) * 16u;
         __builtin_amdgcn_global_load_lds(
             (const void __attribute__((address_space(1)))*)(reinterpret_cast<const char*>(qb) + (size_t)off),
             (void __attribute__((address_space(3)))*)(qstage + i * 512), 16, 0, 0);
@@ -236,22 +258,29 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         const int t2 = wave * kDmaPerWave + i;
         const int r = (t2 >> 1) * kRowsPerDma + dma_row;
         // V of a leaf tile is read row-wise like K (no transposing read), so it takes K's swizzle
-        dma_leaf[i] = (uint32_t)k_chunk<D>(r, dma_slot) * 16u;
-        dma_flip[i] = (t2 & 1) ? ((uint32_t)v16_chunk<D>(r, dma_slot) * 16u) ^ dma_leaf[i] : 0u;
+        if constexpr (KV8) {   // staged as stored (chunk = slot); the swizzle is applied when the tile is widened
+            dma_leaf[i] = 0u;
+            dma_flip[i] = 0u;
+        } else {
+            dma_leaf[i] = (uint32_t)k_chunk<D>(r, dma_slot) * 16u;
+            dma_flip[i] = (t2 & 1) ? ((uint32_t)v16_chunk<D>(r, dma_slot) * 16u) ^ dma_leaf[i] : 0u;
+        }
     }
     auto issue_rows = [&](int t, int slot, const int (&rows)[kRowGroups]) {
-        T* dst_tile = ring + slot * 2 * kTileElems;
+        unsigned char* dst_tile = KV8 ? stage8 + slot * kStageBytes : reinterpret_cast<unsigned char*>(ring + slot * 2 * kTileElems);
+        constexpr int kHalf = KV8 ? kStageBytes / 2 : kTileElems * 2;   // bytes from the K part to the V part
         const uint32_t anc_tile = t < kLeafTiles ? 0u : 0xffffffffu;
 #pragma unroll
         for (int i = 0; i < kDmaPerWave; ++i) {
             const int t2 = wave * kDmaPerWave + i;
             const int u = t2 >> 1;
             const bool is_v = t2 & 1;
-            const uint32_t off = (uint32_t)rows[i >> 1] * (uint32_t)(D * sizeof(T)) + (dma_leaf[i] ^ (dma_flip[i] & anc_tile));
+            const uint32_t off = (uint32_t)rows[i >> 1] * (uint32_t)kKvRowBytes +
+                                 (KV8 ? (uint32_t)dma_slot * 16u : dma_leaf[i] ^ (dma_flip[i] & anc_tile));
             const char* src = reinterpret_cast<const char*>(is_v ? vb : kb) + (size_t)off;
             __builtin_amdgcn_global_load_lds(
                 (const void __attribute__((address_space(1)))*)src,
-                (void __attribute__((address_space(3)))*)(dst_tile + (is_v ? kTileElems : 0) + u * 512),
+                (void __attribute__((address_space(3)))*)(dst_tile + (is_v ? kHalf : 0) + u * 1024),
                 16, 0, 0);
         }
     };
@@ -358,15 +387,90 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     // then refill the slots that barrier freed.
     int issued = n_spec, issue_slot = n_spec, consumed = 0, slot = 0;   // n_spec < stages
     if (!tree) issued = consumed = kLeafTiles;   // no tree part: the list starts behind the leaf tiles
-    auto refill = [&]() {
-        while (issued < total_tiles && issued < consumed + stages) {
+    auto refill_to = [&](int limit) {   // requests tiles up to (not including) list position `limit`
+        while (issued < total_tiles && issued < limit) {
             issue(issued, issue_slot);
             ++issued;
             issue_slot = issue_slot + 1 == stages ? 0 : issue_slot + 1;
         }
     };
+    auto refill = [&]() { refill_to(consumed + stages); };
+    // 8-bit K/V: tile t of the list waits in staging slot t % stages and is widened into 16-bit tile
+    // t % 2.  Eight values (8 bytes) per piece: K rows land in the K swizzle, V rows of ancestor
+    // and prefix tiles in the swizzle of the transposing read, V rows of leaf tiles in K's.
+    int widened = consumed;     // tiles widened so far (by this wave's share; complete behind the next barrier)
+    auto widen = [&](int t) {
+        if constexpr (KV8) {
+            const unsigned char* src = stage8 + (t % stages) * kStageBytes;
+            T* dst = ring + (t & 1) * 2 * kTileElems;
+            constexpr int kPieces = 2 * kTileN * D / 8;        // K pieces, then V pieces
+            constexpr int kPerThread = kPieces / kThreads;     // (a power of two)
+            static_assert(kPerThread * kThreads == kPieces, "pieces split evenly over the threads");
+            const bool leaf_tile = t < kLeafTiles;
+            // two pieces are requested before the first one is widened (more would not fit the registers
+            // of the 64-row blocks): one LDS round trip per pair
+            constexpr int kBatch = kPerThread >= 2 ? 2 : 1;
+            static_assert(kPerThread % kBatch == 0, "pieces come in pairs (or one per thread)");
+#pragma unroll 1
+            for (int i0 = 0; i0 < kPerThread; i0 += kBatch) {
+                u32x2 raw[kBatch];
+#pragma unroll
+                for (int i = 0; i < kBatch; ++i) {
+                    const int piece = (i0 + i) * kThreads + tid;
+                    const int is_v = piece >= kPieces / 2 ? 1 : 0;
+                    const int idx = piece - is_v * (kPieces / 2);
+                    raw[i] = lds_read_b64(lds_addr(src + is_v * (kStageBytes / 2) + (idx / kCpr) * D + (idx % kCpr) * 8));
+                }
+                lds_wait();
+#pragma unroll
+                for (int i = 0; i < kBatch; ++i) {
+                    const int piece = (i0 + i) * kThreads + tid;
+                    const int is_v = piece >= kPieces / 2 ? 1 : 0;
+                    const int idx = piece - is_v * (kPieces / 2);
+                    const int row = idx / kCpr, c = idx % kCpr;
+                    lds_tie(raw[i]);
+                    const uint32_t lo = raw[i][0], hi = raw[i][1];
+                    u32x4 wide;
+                    if constexpr (BF16) {
+                        wide[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false));
+                        wide[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true));
+                        wide[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false));
+                        wide[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true));
+                    } else {
+                        wide[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, false));
+                        wide[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, true));
+                        wide[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, false));
+                        wide[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, true));
+                    }
+                    const int chunk = (is_v && !leaf_tile) ? v16_chunk<D>(row, c) : k_chunk<D>(row, c);
+                    lds_write_b128(lds_addr(dst + is_v * kTileElems + row * D + chunk * 8), wide);
+                }
+            }
+        }
+    };
     bool all_landed = false;   // every tile of the list is in LDS and every wave knows it
     auto begin_step = [&](int n) {
+        if constexpr (KV8) {
+            // (n == 1) Tile `consumed` must be widened and visible; tile consumed + 1 is widened during
+            // this step.  A staging slot is free again once its tile has been widened by everyone,
+            // i.e. behind the barrier after that: the slots of tiles up to `consumed` here.
+            if (widened == consumed) {   // first step: nothing widened yet
+                wait_tiles_outstanding<kDmaPerWave>(max(issued - consumed - 1, 0));
+                ring_barrier();
+                widen(consumed);
+                widened = consumed + 1;
+            }
+            const bool more = consumed + 1 < total_tiles;
+            if (more && issued < consumed + 2) refill_to(consumed + 2);   // (a ring of one slot)
+            if (more) wait_tiles_outstanding<kDmaPerWave>(max(issued - consumed - 2, 0));
+            ring_barrier();
+            refill_to(consumed + 1 + stages);
+            if (more) {
+                widen(consumed + 1);
+                widened = consumed + 2;
+            }
+            return;
+        }
         if (kDShare && all_landed) return;
         if (kDShare && issued == total_tiles && consumed >= kLeafTiles) {
             // short list, the last tiles are in flight: wait for all of them once instead of
@@ -392,6 +496,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         if (slot >= stages) slot -= stages;
     };
     auto tile_ptr = [&](int i) {   // K tile of the i-th tile of the current step; V follows it
+        if constexpr (KV8) return ring + ((consumed + i) & 1) * 2 * kTileElems;
         int sl = slot + i;
         if (sl >= stages) sl -= stages;
         return ring + sl * 2 * kTileElems;
@@ -447,7 +552,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
 #pragma unroll
             for (int dt = 0; dt < kOTiles; ++dt) lds_tie(vraw[dt]);
             if (leaf_ok) {
-                m_i = dot * p.scale_log2e;
+                m_i = dot * sc;
                 l_i = g == 0 ? 1.f : 0.f;
 #pragma unroll
                 for (int dt = 0; dt < kOTiles; ++dt) {
@@ -549,7 +654,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
             const float neg_m = m_i == -INFINITY ? 0.f : -m_i;
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
-                pw[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[r], p.scale_log2e, neg_m));
+                pw[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[r], sc, neg_m));
                 rowsum += pw[r];
             }
         }
@@ -558,7 +663,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
             float mx_raw = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
                                  fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
             mx_raw = max_quarters(mx_raw);
-            const float mx = mx_raw * p.scale_log2e;   // the scale is positive here
+            const float mx = mx_raw * sc;   // the scale is positive here
             // raise only rows that would otherwise keep a weight above 2^kRescaleSlack
             const bool raise = mx > m_i + kRescaleSlack || (m_i == -INFINITY && mx > -INFINITY);
             const float alpha = raise ? __builtin_amdgcn_exp2f(m_i - mx) : 1.f;   // exp2(-inf) = 0
@@ -572,7 +677,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
             rowsum = 0.f;
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
-                pw[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[r], p.scale_log2e, neg_m));
+                pw[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[r], sc, neg_m));
                 rowsum += pw[r];
             }
         }
@@ -621,7 +726,8 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     auto finish = [&](auto& vals, int col0, unsigned char* stage, bool write_lse) {
         constexpr int kTilesHere = (int)(sizeof(vals) / sizeof(vals[0]));
         const float l_tot = sum_quarters(l_i);
-        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+        float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+        if (KV8 && p.v_scale) inv *= p.v_scale[hz];   // O was accumulated on the stored V values
         if (write_lse) {
             // the row number is derived again from an opaque copy: kept from the start-up it
             // would occupy a register pair through the whole kernel
@@ -763,8 +869,8 @@ int launch_ks(const AttnParams& p, int sub_shift, hipStream_t stream) {
                            stream, p, stages, early, shift_arg);
     }
     FSTA_HIP_OK(hipGetLastError());
-    note_launch({"attn_mfma16_kernel", BF16 ? "true" : "false", {D, M, SPLIT ? 1 : 0, KS, p.key_splits > 1 ? 1 : 0}, 5,
-                 0x14u, sub_shift, early});
+    note_launch({"attn_mfma16_kernel", BF16 ? "true" : "false", {D, M, SPLIT ? 1 : 0, KS, p.key_splits > 1 ? 1 : 0, 0}, 6,
+                 0x34u, sub_shift, early});
     return FSTA_OK;
 }
 
@@ -813,7 +919,58 @@ int launch_d(const AttnParams& p, int head_dim, hipStream_t stream) {
     return fail(FSTA_EUNSUPPORTED, "matrix-core kernel: head_dim=%d", head_dim);
 }
 
+// 8-bit K/V: one wave per group of 16 rows, whole blocks, no key runs.
+template <bool BF16, int D, int M>
+int launch_kv8(const AttnParams& p, hipStream_t stream) {
+    constexpr bool kSplitP = BF16;
+    const int tiles = M / 32 + anc_tile_capacity(p.max_anc) + (p.prefix + kTileN - 1) / kTileN;
+    int stages = tiles < 2 ? 2 : (tiles > kMaxStages ? kMaxStages : tiles);
+    const size_t plan_bytes = (size_t)plan_layout(M, p.max_anc).block_words * 4;
+    auto lds_for = [&](int st) { return (size_t)2 * 2 * kTileN * D * 2 + (size_t)st * 2 * kTileN * D + plan_bytes; };
+    size_t lds = lds_for(stages);
+    while (lds > 160 * 1024 && stages > 2) lds = lds_for(--stages);
+    constexpr size_t kEpilogueBytes = (size_t)(M / 16) * 16 * (D * 2 + 16);
+    if (lds < kEpilogueBytes) lds = kEpilogueBytes;
+    if (lds > 160 * 1024)
+        return fail(FSTA_EUNSUPPORTED, "8-bit K/V: max_ancestors=%d needs %zu bytes of LDS (limit 163840)", p.max_anc, lds);
+    const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
+    const unsigned grid = (unsigned)(kXcds * slices_per_xcd * p.nb);
+    const bool linear_grid = p.nb > 65535 || slices_per_xcd > 65535;
+    const dim3 grid3 = linear_grid ? dim3(grid) : dim3((unsigned)kXcds, (unsigned)p.nb, (unsigned)slices_per_xcd);
+    if (lds > 64 * 1024) {
+        const int rc = allow_full_lds<&attn_mfma16_kernel<BF16, D, M, kSplitP, 1, false, true>>();
+        if (rc != FSTA_OK) return rc;
+    }
+    hipLaunchKernelGGL((attn_mfma16_kernel<BF16, D, M, kSplitP, 1, false, true>), grid3, dim3(M * 4), lds, stream, p,
+                       stages, 0, linear_grid ? 0x100 : 0);
+    FSTA_HIP_OK(hipGetLastError());
+    note_launch({"attn_mfma16_kernel", BF16 ? "true" : "false", {D, M, kSplitP ? 1 : 0, 1, 0, 1}, 6, 0x34u, 0, 0});
+    return FSTA_OK;
+}
+
+template <bool BF16, int D>
+int launch_kv8_m(const AttnParams& p, hipStream_t stream) {
+    switch (p.block_m) {
+        case 32: return launch_kv8<BF16, D, 32>(p, stream);
+        case 64: return launch_kv8<BF16, D, 64>(p, stream);
+        case 128: return launch_kv8<BF16, D, 128>(p, stream);
+    }
+    return fail(FSTA_EUNSUPPORTED, "8-bit K/V: block_m=%d (supported: 32, 64, 128)", p.block_m);
+}
+
 }  // namespace
+
+int launch_attention_mfma16_kv8(const AttnParams& p, int dtype, int head_dim, hipStream_t stream) {
+    if ((uint64_t)p.nk * (uint64_t)head_dim > 0xffffffffull || !p.plan)
+        return fail(FSTA_EUNSUPPORTED, "8-bit K/V needs a block plan and slices below 4 GiB");
+    const bool bf16 = dtype == FSTA_BF16;
+    if (dtype != FSTA_BF16 && dtype != FSTA_F16) return fail(FSTA_EUNSUPPORTED, "8-bit K/V: q must be float16 or bfloat16");
+    switch (head_dim) {
+        case 64: return bf16 ? launch_kv8_m<true, 64>(p, stream) : launch_kv8_m<false, 64>(p, stream);
+        case 128: return bf16 ? launch_kv8_m<true, 128>(p, stream) : launch_kv8_m<false, 128>(p, stream);
+    }
+    return fail(FSTA_EUNSUPPORTED, "8-bit K/V: head_dim=%d (supported: 64, 128)", head_dim);
+}
 
 int launch_attention_mfma16(const AttnParams& p, int dtype, int head_dim, bool fast_pv, hipStream_t stream) {
     // the gathers address a (batch, head) slice of K or V with 32-bit byte offsets

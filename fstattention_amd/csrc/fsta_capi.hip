@@ -16,7 +16,7 @@ int fail(int code, const char* fmt, ...) {
     return code;
 }
 
-static thread_local LaunchNote g_note = {nullptr, "", {0, 0, 0, 0, 0}, 0, 0u, 0, 0};
+static thread_local LaunchNote g_note = {nullptr, "", {0, 0, 0, 0, 0, 0}, 0, 0u, 0, 0};
 static thread_local char g_note_text[192] = "";
 
 void note_launch(const LaunchNote& note) { g_note = note; }
@@ -163,6 +163,7 @@ extern "C" int fsta_attention_fwd_ws(const void* q, const void* k, const void* v
     p.scale_log2e = sm_scale * kLog2e;
     p.key_splits = 1; p.split_tiles = 0; p.part_o = nullptr; p.part_lse = nullptr;
     p.share_tiles = (flags & FSTA_FLAG_SHARE_TILES) ? 1 : 0;
+    p.k_scale = nullptr; p.v_scale = nullptr;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (workspace && p.plan) {
@@ -195,4 +196,51 @@ extern "C" int fsta_attention_fwd_ws(const void* q, const void* k, const void* v
         if (rc != FSTA_EUNSUPPORTED) return rc;
     }
     return launch_attention_generic(p, dtype, head_dim, s);
+}
+
+extern "C" int fsta_attention_fwd_kv8(const void* q, const void* k8, const void* v8, const float* k_scale,
+                                      const float* v_scale, void* o, float* lse, const uint32_t* block_plan,
+                                      int32_t plan_key_shift, int32_t batch, int32_t heads, int32_t nq, int32_t nk,
+                                      int32_t head_dim, int32_t dtype, int32_t out_dtype, int32_t block_m,
+                                      int32_t max_ancestors, int32_t num_blocks, float sm_scale, void* stream) {
+    if (batch < 0 || heads < 0 || nq < 0 || nk < nq)
+        return fail(FSTA_EINVAL, "fsta_attention_fwd_kv8: batch=%d heads=%d nq=%d nk=%d (need nk >= nq >= 0)", batch,
+                    heads, nq, nk);
+    if (dtype != FSTA_F16 && dtype != FSTA_BF16)
+        return fail(FSTA_EINVAL, "fsta_attention_fwd_kv8: dtype=%d (q must be float16 or bfloat16)", dtype);
+    if (out_dtype != dtype && out_dtype != FSTA_F32)
+        return fail(FSTA_EINVAL, "fsta_attention_fwd_kv8: out_dtype=%d must equal dtype=%d or be float32", out_dtype, dtype);
+    if (head_dim != 64 && head_dim != 128)
+        return fail(FSTA_EUNSUPPORTED, "fsta_attention_fwd_kv8: head_dim=%d (supported: 64, 128)", head_dim);
+    if (!plan_block_size_ok(block_m))
+        return fail(FSTA_EUNSUPPORTED, "fsta_attention_fwd_kv8: block_m=%d (supported: 32, 64, 128)", block_m);
+    if (max_ancestors < 1) return fail(FSTA_EINVAL, "fsta_attention_fwd_kv8: max_ancestors=%d", max_ancestors);
+    if (num_blocks != (nq + block_m - 1) / block_m)
+        return fail(FSTA_EINVAL, "fsta_attention_fwd_kv8: num_blocks=%d but ceil(nq=%d / block_m=%d) = %d", num_blocks, nq,
+                    block_m, (nq + block_m - 1) / block_m);
+    if (!(sm_scale > 0.f)) return fail(FSTA_EUNSUPPORTED, "fsta_attention_fwd_kv8: sm_scale must be positive");
+    const int64_t slices = (int64_t)batch * heads;
+    if (slices > 65535) return fail(FSTA_EUNSUPPORTED, "fsta_attention_fwd_kv8: batch*heads=%lld > 65535", (long long)slices);
+    if (slices == 0 || nq == 0) return FSTA_OK;
+    if (!q || !k8 || !v8 || !o || !block_plan) return fail(FSTA_EINVAL, "fsta_attention_fwd_kv8: null pointer");
+    if (misaligned(q, 16) || misaligned(k8, 16) || misaligned(v8, 16) || misaligned(o, 16) || misaligned(block_plan, 16))
+        return fail(FSTA_EINVAL, "fsta_attention_fwd_kv8: q, k8, v8, o and block_plan must be 16-byte aligned");
+    if (misaligned(k_scale, 4) || misaligned(v_scale, 4) || misaligned(lse, 4))
+        return fail(FSTA_EINVAL, "fsta_attention_fwd_kv8: k_scale, v_scale and lse must be 4-byte aligned");
+    if (plan_key_shift < 0 || plan_key_shift > nk)
+        return fail(FSTA_EINVAL, "fsta_attention_fwd_kv8: plan_key_shift=%d outside [0, nk=%d]", plan_key_shift, nk);
+    AttnParams p;
+    p.q = q; p.k = k8; p.v = v8; p.o = o; p.lse = lse;
+    p.ancestor_idx = nullptr; p.mask_bits = nullptr; p.anc_count = nullptr; p.leaf_idx = nullptr;
+    p.plan = block_plan; p.key_shift = plan_key_shift;
+    p.nq = nq; p.nk = nk; p.prefix = nk - nq;
+    p.block_m = block_m; p.max_anc = max_ancestors; p.mask_words = fsta_mask_words(max_ancestors);
+    p.nb = num_blocks;
+    p.heads_total = (int32_t)slices;
+    p.out_f32 = (out_dtype == FSTA_F32) ? 1 : 0;
+    p.scale_log2e = sm_scale * kLog2e;
+    p.key_splits = 1; p.split_tiles = 0; p.part_o = nullptr; p.part_lse = nullptr;
+    p.share_tiles = 0;
+    p.k_scale = k_scale; p.v_scale = v_scale;
+    return launch_attention_mfma16_kv8(p, dtype, head_dim, static_cast<hipStream_t>(stream));
 }

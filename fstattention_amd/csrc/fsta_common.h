@@ -57,6 +57,10 @@ struct AttnParams {
     int32_t share_tiles;          // tuning: wave pairs of a row group always share the tiles, never the head dimension
     float* part_o;
     float* part_lse;
+    // 8-bit K/V (fsta_attention_fwd_kv8): k and v hold OCP e4m3 bytes; one float32 scale per
+    // (batch, head) slice each, or null for 1
+    const float* k_scale;
+    const float* v_scale;
 };
 
 // true when a non-null pointer is not a multiple of `bytes` (null pointers are judged elsewhere)
@@ -91,11 +95,11 @@ int allow_full_lds() {
 }
 
 // Which attention kernel the calling thread launched last (fsta_last_attention_kernel): the kernel's
-// name and up to six template arguments, kept as numbers and turned into text only when asked for.
+// name and up to seven template arguments, kept as numbers and turned into text only when asked for.
 struct LaunchNote {
     const char* kernel;   // string literal
     const char* first;    // first template argument as text, e.g. "true" or "float"
-    int args[5];
+    int args[6];
     int n_args;
     unsigned bool_args;   // bit i: args[i] is a bool template argument
     int half_blocks, early_start;   // launch options of the narrow matrix-core kernel
@@ -108,6 +112,7 @@ int launch_attention_mfma(const AttnParams& p, int dtype, int head_dim, bool fas
                           hipStream_t stream);
 int launch_attention_mfma16(const AttnParams& p, int dtype, int head_dim, bool fast_pv,
                             hipStream_t stream);
+int launch_attention_mfma16_kv8(const AttnParams& p, int dtype, int head_dim, hipStream_t stream);
 bool mfma_supported(int dtype, int head_dim, int block_m);
 // joins `splits` partial results (layout of AttnParams::part_o / part_lse) into o (and lse, may be null)
 int launch_merge_splits(const float* part_o, const float* part_lse, int splits, int64_t rows, int head_dim,

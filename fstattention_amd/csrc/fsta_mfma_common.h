@@ -154,6 +154,9 @@ __device__ __forceinline__ uint32_t global_read_b32(const void* ptr) {
 __device__ __forceinline__ void lds_write_b32(uint32_t addr, uint32_t value) {
     asm volatile("ds_write_b32 %0, %1" : : "v"(addr), "v"(value) : "memory");
 }
+__device__ __forceinline__ void lds_write_b128(uint32_t addr, u32x4 value) {
+    asm volatile("ds_write_b128 %0, %1" : : "v"(addr), "v"(value) : "memory");
+}
 // Waits for every outstanding LDS access of this wave.
 __device__ __forceinline__ void lds_wait() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 // Orders every later use of `x` behind the preceding lds_wait().

@@ -213,6 +213,26 @@ int fsta_attention_fwd_ws(const void* q, const void* k, const void* v, void* o, 
                           void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * The same operation on K and V stored as 8-bit floats: k8, v8 [batch, heads, nk,
+ * head_dim] bytes in the OCP e4m3 format ("float8_e4m3fn": 1 sign, 4 exponent, 3
+ * mantissa bits, no infinities), with one float32 scale per (batch, head) slice
+ * each (k_scale, v_scale [batch*heads], NULL = 1): the keys are k8 * k_scale, the
+ * values v8 * v_scale.  q and o stay 16-bit (dtype FSTA_F16 / FSTA_BF16; out_dtype
+ * = dtype or FSTA_F32) and all arithmetic is that of fsta_attention_fwd: the rows
+ * are widened exactly in the kernel, so the result is fsta_attention_fwd's on the
+ * widened K and V.  Half the K/V bytes travel.  No counterpart in the reference
+ * (16-bit tensors only).  Needs the block plan (no index lists are read);
+ * head_dim 64 or 128, block_m 32, 64 or 128, sm_scale > 0; other shapes are
+ * refused with FSTA_EUNSUPPORTED.  Alignment: q, k8, v8, o, block_plan 16 bytes;
+ * k_scale, v_scale, lse 4 bytes.
+ */
+int fsta_attention_fwd_kv8(const void* q, const void* k8, const void* v8, const float* k_scale,
+                           const float* v_scale, void* o, float* lse, const uint32_t* block_plan,
+                           int32_t plan_key_shift, int32_t batch, int32_t heads, int32_t nq, int32_t nk,
+                           int32_t head_dim, int32_t dtype, int32_t out_dtype, int32_t block_m,
+                           int32_t max_ancestors, int32_t num_blocks, float sm_scale, void* stream);
+
+/*
  * parent[n_nodes] int64 (parent[i] < i, -1 for roots) -> level_lookup [n_nodes]
  * and lineage [n_nodes, width] in the layout of utils.py:66-75 (strict ancestor
  * a of i at lineage[i, level(a)], -1 elsewhere).  `status` (zero on entry) gets
