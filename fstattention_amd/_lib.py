@@ -90,6 +90,24 @@ def load():
     return lib
 
 
+TORCH_OPS_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_fsta_torch.so")
+_ops = None
+
+
+def load_torch_ops():
+    """``torch.ops.fsta`` (the operator registration of ``csrc/fsta_torch_binding.cpp``), loaded once."""
+    global _ops
+    if _ops is not None:
+        return _ops
+    load()
+    if not os.path.exists(TORCH_OPS_PATH):
+        raise ImportError(f"{TORCH_OPS_PATH} is missing: build it with `python -m fstattention_amd.build`")
+    import torch
+    torch.ops.load_library(TORCH_OPS_PATH)
+    _ops = torch.ops.fsta
+    return _ops
+
+
 def check(code: int):
     if code != OK:
         raise FstaError(code, load().fsta_last_error().decode("utf-8", "replace"))

@@ -202,92 +202,41 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
     Lq, Lk, Lv = q.shape[-1], k.shape[-1], v.shape[-1]
     assert Lq == Lk and Lk == Lv
     assert Lk in {16, 32, 64, 128}
-    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
-        raise ValueError("q, k, v must be [batch, heads, seq, head_dim]")
-    if not (q.is_cuda and k.is_cuda and v.is_cuda):
-        raise ValueError("fst_attention runs on the GPU only (no CPU fallback); move q/k/v to 'cuda'")
-    if not (q.device == k.device == v.device == ancestor_idx.device == leaf_idx.device):
-        raise ValueError("all tensors must live on the same device")
-    kv8 = k.dtype == _FP8
-    if kv8:
-        if v.dtype != _FP8 or q.dtype not in (torch.float16, torch.bfloat16):
-            raise ValueError(f"8-bit K/V: k and v must both be float8_e4m3fn and q float16/bfloat16, got "
-                             f"{q.dtype}, {k.dtype}, {v.dtype}")
-        if fast_pv or generic or wide_waves or key_splits or share_tiles:
-            raise ValueError("8-bit K/V has one kernel: fast_pv, generic, wide_waves, key_splits and share_tiles do not apply")
-    elif q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
-        raise ValueError(f"q/k/v must share one dtype of float32/float16/bfloat16, got "
-                         f"{q.dtype}, {k.dtype}, {v.dtype}")
-    if (k_scale is not None or v_scale is not None) and not kv8:
-        raise ValueError("k_scale / v_scale belong to 8-bit K/V (float8_e4m3fn k and v)")
-    if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
-        raise ValueError("q, k, v must be contiguous")
-    Z, H, Nq, D = q.shape
-    if k.shape[:2] != (Z, H) or v.shape != k.shape:
-        raise ValueError(f"k/v shapes {tuple(k.shape)}/{tuple(v.shape)} do not match q {tuple(q.shape)}")
-    Nk = k.shape[2]
-    if Nk < Nq:
-        raise ValueError(f"k has {Nk} rows, fewer than q's {Nq}")
-    nb = -(-Nq // BLOCK_M)
-    if ancestor_idx.dtype != torch.int64 or leaf_idx.dtype != torch.int64:
-        raise ValueError("ancestor_idx and leaf_idx must be int64")
-    if tuple(ancestor_idx.shape) != (nb, MAX_ANCESTORS):
-        raise ValueError(f"ancestor_idx is {tuple(ancestor_idx.shape)}, expected "
-                         f"(ceil(Nq/BLOCK_M)={nb}, MAX_ANCESTORS={MAX_ANCESTORS})")
-    if tuple(leaf_idx.shape) != (nb, BLOCK_M):
-        raise ValueError(f"leaf_idx is {tuple(leaf_idx.shape)}, expected ({nb}, BLOCK_M={BLOCK_M})")
     if isinstance(ancestor_mask, PackedTreeMask):
-        if (ancestor_mask.block_m, ancestor_mask.max_ancestors) != (BLOCK_M, MAX_ANCESTORS) or \
-                ancestor_mask.mask_bits.shape[0] != nb:
+        if (ancestor_mask.block_m, ancestor_mask.max_ancestors) != (BLOCK_M, MAX_ANCESTORS):
             raise ValueError("packed mask was built for another block size / ancestor count")
-    elif tuple(ancestor_mask.shape) != (nb, BLOCK_M, MAX_ANCESTORS):
-        raise ValueError(f"ancestor_mask is {tuple(ancestor_mask.shape)}, expected "
-                         f"({nb}, {BLOCK_M}, {MAX_ANCESTORS})")
-    out_dtype = out_dtype or q.dtype
-    if out_dtype not in (q.dtype, torch.float32):
-        raise ValueError("out_dtype must be the input dtype or torch.float32")
-
-    lib = _lib.load()
-    ancestor_idx = ancestor_idx.contiguous()
-    leaf_idx = leaf_idx.contiguous()
-    packed = _packed_for(ancestor_idx, ancestor_mask, leaf_idx, Nk)
-    plan_ptr = packed.plan.data_ptr() if packed.plan is not None else None
-    o = torch.empty(q.shape, dtype=out_dtype, device=q.device)
-    # the reference allocates L and drops it (fstattention.py:158-160,181); here it only exists when asked for
-    lse = torch.empty((Z * H, Nq), device=q.device, dtype=torch.float32) if return_lse else None
-    flags = (_lib.FLAG_FAST_PV if fast_pv else 0) | (_lib.FLAG_GENERIC if generic else 0) | \
-        (_lib.FLAG_WIDE_WAVES if wide_waves else 0) | (_lib.flag_key_splits(key_splits) if key_splits else 0) | \
-        (_lib.FLAG_SHARE_TILES if share_tiles else 0)
-    if kv8:
-        for name, scale in (("k_scale", k_scale), ("v_scale", v_scale)):
-            if scale is not None and (scale.dtype != torch.float32 or scale.numel() != Z * H or
-                                      scale.device != q.device or not scale.is_contiguous()):
-                raise ValueError(f"{name} must be a contiguous float32 tensor of {Z * H} entries on {q.device}")
-        if plan_ptr is None:
-            raise ValueError(f"8-bit K/V needs BLOCK_M of 32, 64 or 128 (got {BLOCK_M})")
-        with _on_device(q.device):
-            _lib.check(lib.fsta_attention_fwd_kv8(
-                q.data_ptr(), k.data_ptr(), v.data_ptr(), k_scale.data_ptr() if k_scale is not None else None,
-                v_scale.data_ptr() if v_scale is not None else None, o.data_ptr(),
-                lse.data_ptr() if return_lse else None, plan_ptr, packed.key_shift, Z, H, Nq, Nk, D,
-                _DTYPES[q.dtype], _DTYPES[out_dtype], BLOCK_M, MAX_ANCESTORS, nb, float(sm_scale),
-                _stream_ptr(q.device)))
-        return (o, lse) if return_lse else o
-    # a shared prefix may be worth cutting into key runs: the library says how much workspace that takes
-    work, work_bytes = None, 0
-    if Nk > Nq:
-        work_bytes = lib.fsta_attention_workspace_bytes(Z, H, Nq, Nk, D, _DTYPES[q.dtype], BLOCK_M,
-                                                        MAX_ANCESTORS, float(sm_scale), flags)
-        if work_bytes:
-            work = torch.empty((work_bytes,), dtype=torch.uint8, device=q.device)
-    with _on_device(q.device):
-        _lib.check(lib.fsta_attention_fwd_ws(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr() if return_lse else None,
-            ancestor_idx.data_ptr(), packed.mask_bits.data_ptr(), packed.anc_count.data_ptr(),
-            leaf_idx.data_ptr(), plan_ptr, packed.key_shift, Z, H, Nq, Nk, D, _DTYPES[q.dtype], _DTYPES[out_dtype],
-            BLOCK_M, MAX_ANCESTORS, nb, float(sm_scale), flags,
-            work.data_ptr() if work is not None else None, work_bytes, _stream_ptr(q.device)))
+        packed = ancestor_mask
+    else:
+        if ancestor_mask.dim() != 3 or ancestor_mask.shape[1] != BLOCK_M or ancestor_mask.shape[2] != MAX_ANCESTORS or \
+                ancestor_mask.shape[0] != ancestor_idx.shape[0]:
+            raise ValueError(f"ancestor_mask is {tuple(ancestor_mask.shape)}, expected "
+                             f"({ancestor_idx.shape[0]}, {BLOCK_M}, {MAX_ANCESTORS})")
+        if q.dim() != 4 or k.dim() != 4:
+            raise ValueError("q, k, v must be [batch, heads, seq, head_dim]")
+        packed = _packed_for(ancestor_idx, ancestor_mask, leaf_idx, k.shape[2])
+    out_code = _DTYPES.get(out_dtype or q.dtype)
+    if out_code is None:
+        raise ValueError("q must be float32/float16/bfloat16 and out_dtype the input dtype or torch.float32")
+    flags = 0
+    if fast_pv or generic or wide_waves or key_splits or share_tiles:
+        flags = (_lib.FLAG_FAST_PV if fast_pv else 0) | (_lib.FLAG_GENERIC if generic else 0) | \
+            (_lib.FLAG_WIDE_WAVES if wide_waves else 0) | (_lib.flag_key_splits(key_splits) if key_splits else 0) | \
+            (_lib.FLAG_SHARE_TILES if share_tiles else 0)
+    # everything else (the remaining checks, o and L, the workspace of key runs, the launch on the current stream)
+    # happens in the registered operator, csrc/fsta_torch_binding.cpp
+    o, lse = (_OPS or _ops()).attention_fwd(q, k, v, ancestor_idx, packed.mask_bits, packed.anc_count, leaf_idx, packed.plan,
+                                            packed.key_shift, float(sm_scale), BLOCK_M, MAX_ANCESTORS, out_code, return_lse, flags,
+                                            k_scale, v_scale)
     return (o, lse) if return_lse else o
+
+
+_OPS = None
+
+
+def _ops():
+    global _OPS
+    _OPS = _lib.load_torch_ops()
+    return _OPS
 
 
 def shift_for_prefix(ancestor_idx: torch.Tensor, leaf_idx: torch.Tensor, prefix: int,

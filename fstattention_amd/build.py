@@ -112,5 +112,31 @@ def build_library(verbose: bool = True, jobs: int | None = None) -> str:
     return LIB_PATH
 
 
+TORCH_OPS_PATH = os.path.join(PKG_DIR, "_fsta_torch.so")
+
+
+def build_torch_ops(verbose: bool = True) -> str:
+    """Compiles ``csrc/fsta_torch_binding.cpp`` (host code: the ``torch.ops.fsta`` registration on top of
+    the C ABI) with the host compiler against this interpreter's torch and links it to ``libfsta.so``."""
+    import torch
+    from torch.utils import cpp_extension as ce
+    cxx = os.environ.get("CXX") or shutil.which("g++")
+    if not cxx:
+        raise RuntimeError("g++ not found (set CXX)")
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    includes = [f"-I{d}" for d in ce.include_paths("cuda")]
+    tmp = TORCH_OPS_PATH + ".tmp"
+    _run([cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+          f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", "-Wno-deprecated-declarations",
+          *includes, os.path.join(CSRC, "fsta_torch_binding.cpp"), "-o", tmp,
+          f"-L{torch_lib}", "-lc10", "-ltorch_cpu", "-ltorch_hip", "-lc10_hip", "-ltorch",
+          f"-L{PKG_DIR}", "-l:libfsta.so", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}"])
+    os.replace(tmp, TORCH_OPS_PATH)
+    if verbose:
+        print(f"built {TORCH_OPS_PATH} ({os.path.getsize(TORCH_OPS_PATH)} bytes)")
+    return TORCH_OPS_PATH
+
+
 if __name__ == "__main__":
     build_library()
+    build_torch_ops()
