@@ -12,6 +12,15 @@ OK, EINVAL, EUNSUPPORTED, EHIP = 0, -1, -2, -3
 FLAG_FAST_PV, FLAG_GENERIC, FLAG_WIDE_WAVES, FLAG_SHARE_TILES = 1, 2, 4, 8
 
 
+DFS_ORDER_MAX_NODES = 131072
+DFS_ORDER_STATIC_MAX_NODES = 16384
+
+
+def dfs_order_workspace_ints(n: int) -> int:
+    """FSTA_DFS_ORDER_WORKSPACE_INTS(n): int32 entries of scratch fsta_dfs_order wants for n nodes."""
+    return 6 * int(n) + 8
+
+
 def flag_key_splits(n: int) -> int:
     """FSTA_FLAG_KEY_SPLITS(n): force n runs of prefix keys (1 = never split, 0 = library decides)."""
     return (int(n) & 0xFF) << 8

@@ -16,10 +16,10 @@
 namespace fsta {
 namespace {
 
-// Scratch of fsta_dfs_order_static: subtree sizes and sibling offsets of one tree.  Every GPU the
-// library runs on holds its own copy of this array (128 KiB) at its own address until the process
+// Scratch of fsta_dfs_order_static: subtree sizes, sibling offsets and child lists of one tree.  Every GPU the
+// library runs on holds its own copy of this array (384 KiB) at its own address until the process
 // ends; in host code the name below is only a handle for hipGetSymbolAddress, never an address.
-static __device__ __align__(256) int32_t scratch[2 * FSTA_DFS_ORDER_STATIC_MAX_NODES];
+static __device__ __align__(256) int32_t scratch[FSTA_DFS_ORDER_WORKSPACE_INTS(FSTA_DFS_ORDER_STATIC_MAX_NODES)];
 
 constexpr int kMaxDevices = 64;
 int32_t* g_scratch_ptr[kMaxDevices] = {};   // device address of `scratch` on each device, once looked up
@@ -42,110 +42,128 @@ int scratch_on_current_device(int32_t** out) {
 }
 
 constexpr int kOrderThreads = 256;
-constexpr int kSiblingTile = 256;    // candidate siblings staged in LDS per workgroup
 
-__device__ __forceinline__ int32_t load_coherent(const int32_t* p) {
-    // values produced by atomics of other workgroups: read past this CU's L1
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+// ---- trees too large for one workgroup's LDS (up to FSTA_DFS_ORDER_MAX_NODES) ----------------------
+// Six launches of N threads over arrays in device memory (they stay in L2: 4 bytes per node each):
+//   size[i]   every node adds 1 to each ancestor (a walk of depth(i) dependent reads)
+//   kids[p]   number of children; the roots are the children of a virtual node N
+//   first[p]  exclusive prefix sum of kids (one workgroup)
+//   child[]   the children of every parent, next to each other (slot by atomic counter: any order)
+//   off[i]    sum of size[s] over the siblings s that the order visits before i: a scan of the
+//             parent's child list, i.e. work proportional to sum over parents of (children)^2
+//   pre[i]    sum over i and its ancestors of (off + 1), minus 1
+// Work O(N * depth + sum of children^2): linear for the trees of tree decoding (bounded fan-out,
+// depth of tens of levels), and still finite for a star or a chain of 2^17 nodes.
+// Every hop of a walk must go to a smaller id (or to -1), so the walks end whatever the input holds.
+__device__ __forceinline__ int32_t checked_parent(const int64_t* __restrict__ parent, int32_t i) {
+    const int64_t p = parent[i];
+    return (p >= -1 && p < i) ? (int32_t)p : -2;   // -2: malformed entry
 }
 
-__global__ __launch_bounds__(kOrderThreads) void order_init_kernel(int64_t n, int32_t* size, int32_t* off) {
-    const int64_t i = (int64_t)blockIdx.x * kOrderThreads + threadIdx.x;
-    if (i < n) {
-        size[i] = 1;
-        off[i] = 0;
-    }
+__global__ __launch_bounds__(kOrderThreads) void order_init_kernel(int32_t n, int32_t* size, int32_t* kids) {
+    const int32_t i = blockIdx.x * kOrderThreads + threadIdx.x;
+    if (i < n) size[i] = 1;
+    if (i <= n) kids[i] = 0;
 }
 
-// The walks to the root are chains of dependent reads; every workgroup first copies the parent
-// array (as int32; n <= 16384) into LDS so that a hop costs an LDS access, not a trip to L2.
-// Every hop must go to a smaller id (or to -1), so the walks end whatever the input holds.
-__device__ __forceinline__ void stage_parents(const int64_t* __restrict__ parent, int64_t n, int32_t* par_s) {
-    for (int64_t i = threadIdx.x; i < n; i += kOrderThreads) {
-        const int64_t p = parent[i];
-        par_s[i] = (p >= -1 && p < i) ? (int32_t)p : -2;   // -2: malformed entry
-    }
-    __syncthreads();
-}
-
-// Every node adds 1 to each of its ancestors.  All nodes meet at the roots, so the counts are
-// first gathered per workgroup in LDS and only the non-zero sums go to the global array.
-__global__ __launch_bounds__(kOrderThreads) void order_sizes_kernel(const int64_t* __restrict__ parent, int64_t n,
-                                                                    int32_t* size, uint32_t* status) {
-    extern __shared__ int32_t par_s[];       // [n] parents, then [n] counts of this workgroup
-    int32_t* count_s = par_s + n;
-    for (int64_t x = threadIdx.x; x < n; x += kOrderThreads) count_s[x] = 0;
-    stage_parents(parent, n, par_s);
-    const int64_t i = (int64_t)blockIdx.x * kOrderThreads + threadIdx.x;
-    if (i < n) {
-        int32_t p = par_s[i];
-        while (p >= 0) {
-            atomicAdd(&count_s[p], 1);
-            p = par_s[p];
-        }
-        if (p < -1) atomicOr(status, FSTA_PRE_BAD_NODE_ID);
-    }
-    __syncthreads();
-    for (int64_t x = threadIdx.x; x < n; x += kOrderThreads)
-        if (count_s[x]) atomicAdd(&size[x], count_s[x]);
-}
-
-// grid (ceil(n / kOrderThreads), ceil(n / kSiblingTile)): thread i against the candidates of tile y
-__global__ __launch_bounds__(kOrderThreads) void order_siblings_kernel(const int64_t* __restrict__ parent, int64_t n,
-                                                                       int light_first, const int32_t* size,
-                                                                       int32_t* off) {
-    __shared__ int32_t par_s[kSiblingTile];
-    __shared__ int32_t size_s[kSiblingTile];
-    const int i = blockIdx.x * kOrderThreads + threadIdx.x;       // n <= 16384: 32-bit arithmetic throughout
-    const int s0 = blockIdx.y * kSiblingTile;
-    // a sibling has an id above the common parent; with plain index order it also lies below i
-    const int block_last = min((int)(blockIdx.x + 1) * kOrderThreads, (int)n) - 1;
-    if (!light_first && s0 > block_last) return;
-    for (int t = threadIdx.x; t < kSiblingTile; t += kOrderThreads) {
-        const int s = s0 + t;
-        par_s[t] = s < n ? (int32_t)parent[s] : -2;     // -2 never matches
-        size_s[t] = s < n ? load_coherent(size + s) : 0;
-    }
-    __syncthreads();
+__global__ __launch_bounds__(kOrderThreads) void order_sizes_kernel(const int64_t* __restrict__ parent, int32_t n,
+                                                                    int32_t* size, int32_t* kids, uint32_t* status) {
+    const int32_t i = blockIdx.x * kOrderThreads + threadIdx.x;
     if (i >= n) return;
-    const int32_t my_parent = (int32_t)parent[i];
-    const int32_t my_size = load_coherent(size + i);
-    const int count = min(kSiblingTile, (int)n - s0);
-    int32_t acc = 0;
-    if (light_first) {
-        // order key (size, id) packed into one comparison: sizes and ids are below 2^15
-        const int32_t my_key = (my_size << 15) | i;
-#pragma unroll 4
-        for (int t = 0; t < count; ++t) {
-            const int32_t key = (size_s[t] << 15) | (s0 + t);
-            acc += (par_s[t] == my_parent && key < my_key) ? size_s[t] : 0;
+    int32_t a = checked_parent(parent, i);
+    if (a >= -1) atomicAdd(&kids[a >= 0 ? a : n], 1);
+    while (a >= 0) {
+        // neighbouring ids often meet after a few hops: where all lanes of the wave that are still
+        // walking stand on the same node, one of them adds for all (else the adds queue up at the roots)
+        const uint64_t walking = __ballot(true);
+        const int32_t first = __builtin_amdgcn_readfirstlane(a);
+        if (__ballot(a != first) == 0ull) {
+            if ((threadIdx.x & 63) == __ffsll((long long)walking) - 1) atomicAdd(&size[first], __popcll(walking));
+        } else {
+            atomicAdd(&size[a], 1);
         }
-    } else {
-#pragma unroll 4
-        for (int t = 0; t < count; ++t) acc += (par_s[t] == my_parent && s0 + t < i) ? size_s[t] : 0;
+        a = checked_parent(parent, a);
     }
-    if (acc) atomicAdd(&off[i], acc);
+    if (a < -1) atomicOr(status, FSTA_PRE_BAD_NODE_ID);
 }
 
-__global__ __launch_bounds__(kOrderThreads) void order_finish_kernel(const int64_t* __restrict__ parent, int64_t n,
-                                                                     const int32_t* off, int64_t* __restrict__ perm,
+constexpr int kScanThreads = 1024;
+
+// first[p] = kids[0] + ... + kids[p-1] for p = 0 .. n (n + 1 entries), cursor = a copy; one workgroup
+__global__ __launch_bounds__(kScanThreads) void order_scan_kernel(int32_t n, const int32_t* __restrict__ kids,
+                                                                  int32_t* __restrict__ first, int32_t* __restrict__ cursor) {
+    __shared__ int32_t wave_sum[kScanThreads / 64];
+    const int tid = threadIdx.x;
+    const int per = (n + 1 + kScanThreads - 1) / kScanThreads;
+    const int lo = min(tid * per, n + 1), hi = min(lo + per, n + 1);
+    int32_t local = 0;
+    for (int x = lo; x < hi; ++x) local += kids[x];
+    int32_t incl = local;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int32_t up = __shfl_up(incl, d, 64);
+        if ((tid & 63) >= d) incl += up;
+    }
+    if ((tid & 63) == 63) wave_sum[tid >> 6] = incl;
+    __syncthreads();
+    int32_t base = 0;
+    for (int w = 0; w < (tid >> 6); ++w) base += wave_sum[w];
+    int32_t run = base + incl - local;
+    for (int x = lo; x < hi; ++x) {
+        first[x] = run;
+        cursor[x] = run;
+        run += kids[x];
+    }
+}
+
+__global__ __launch_bounds__(kOrderThreads) void order_fill_kernel(const int64_t* __restrict__ parent, int32_t n,
+                                                                   int32_t* cursor, int32_t* __restrict__ child) {
+    const int32_t i = blockIdx.x * kOrderThreads + threadIdx.x;
+    if (i >= n) return;
+    const int32_t p = checked_parent(parent, i);
+    if (p < -1) return;     // (flagged by the size pass; the result is the identity)
+    child[atomicAdd(&cursor[p >= 0 ? p : n], 1)] = i;
+}
+
+__global__ __launch_bounds__(kOrderThreads) void order_offsets_kernel(const int64_t* __restrict__ parent, int32_t n,
+                                                                      int light_first, const int32_t* __restrict__ size,
+                                                                      const int32_t* __restrict__ kids,
+                                                                      const int32_t* __restrict__ first,
+                                                                      const int32_t* __restrict__ child,
+                                                                      int32_t* __restrict__ off) {
+    const int32_t i = blockIdx.x * kOrderThreads + threadIdx.x;
+    if (i >= n) return;
+    const int32_t p = checked_parent(parent, i);
+    int32_t acc = 0;
+    if (p >= -1) {
+        const int32_t pp = p >= 0 ? p : n;
+        const int32_t begin = first[pp], count = kids[pp];
+        // order key (size, id) in one comparison; plain index order compares ids only
+        const int64_t my_key = light_first ? ((int64_t)size[i] << 32) | (uint32_t)i : (int64_t)i;
+        for (int32_t c = 0; c < count; ++c) {
+            const int32_t s = child[begin + c];
+            const int32_t sz = size[s];
+            const int64_t key = light_first ? ((int64_t)sz << 32) | (uint32_t)s : (int64_t)s;
+            acc += key < my_key ? sz : 0;
+        }
+    }
+    off[i] = acc;
+}
+
+__global__ __launch_bounds__(kOrderThreads) void order_finish_kernel(const int64_t* __restrict__ parent, int32_t n,
+                                                                     const int32_t* __restrict__ off, int64_t* __restrict__ perm,
                                                                      int64_t* __restrict__ rank,
                                                                      const uint32_t* status) {
-    extern __shared__ int32_t par_s[];       // [n] parents, then [n] sibling offsets
-    int32_t* off_s = par_s + n;
-    const int64_t i = (int64_t)blockIdx.x * kOrderThreads + threadIdx.x;
+    const int32_t i = blockIdx.x * kOrderThreads + threadIdx.x;
+    if (i >= n) return;
     if (*status) {      // malformed parent array: identity, the caller reads the status word
-        if (i < n) {
-            perm[i] = i;
-            rank[i] = i;
-        }
+        perm[i] = i;
+        rank[i] = i;
         return;
     }
-    for (int64_t x = threadIdx.x; x < n; x += kOrderThreads) off_s[x] = load_coherent(off + x);
-    stage_parents(parent, n, par_s);
-    if (i >= n) return;
     int64_t pre = -1;
-    for (int32_t cur = (int32_t)i; cur >= 0; cur = par_s[cur]) pre += off_s[cur] + 1;
+    for (int32_t cur = i; cur >= 0; cur = checked_parent(parent, cur)) pre += off[cur] + 1;
     perm[pre] = i;
     rank[i] = pre;
 }
@@ -278,8 +296,8 @@ extern "C" int fsta_renumber_parents(const int64_t* parent, const int64_t* rank,
 
 namespace {
 
-// The launches of fsta_dfs_order; `workspace`: 2 * n_nodes int32 of device memory (only trees
-// too large for the single-workgroup kernel touch it).
+// The launches of fsta_dfs_order; `workspace`: FSTA_DFS_ORDER_WORKSPACE_INTS(n_nodes) int32 of device
+// memory (only trees too large for the single-workgroup kernel touch it).
 int dfs_order_launch(const int64_t* parent, int64_t n_nodes, int32_t light_first, int64_t* perm, int64_t* rank,
                      int32_t* workspace, uint32_t* status, hipStream_t s) {
     if (n_nodes <= kSmallMaxNodes) {
@@ -293,24 +311,22 @@ int dfs_order_launch(const int64_t* parent, int64_t n_nodes, int32_t light_first
         FSTA_HIP_OK(hipGetLastError());
         return FSTA_OK;
     }
-    int32_t* size = workspace;
-    int32_t* off = workspace + n_nodes;
-    const unsigned blocks = (unsigned)((n_nodes + kOrderThreads - 1) / kOrderThreads);
-    const unsigned tiles = (unsigned)((n_nodes + kSiblingTile - 1) / kSiblingTile);
-    const size_t lds_parents = (size_t)n_nodes * sizeof(int32_t);
-    if (2 * lds_parents > 64 * 1024) {
-        int rc = allow_full_lds<&order_sizes_kernel>();
-        if (rc == FSTA_OK) rc = allow_full_lds<&order_finish_kernel>();
-        if (rc != FSTA_OK) return rc;
-    }
-    // (size and off are set by a kernel: everything of an earlier call is overwritten)
-    hipLaunchKernelGGL(order_init_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, n_nodes, size, off);
-    hipLaunchKernelGGL(order_sizes_kernel, dim3(blocks), dim3(kOrderThreads), 2 * lds_parents, s, parent, n_nodes,
-                       size, status);
-    hipLaunchKernelGGL(order_siblings_kernel, dim3(blocks, tiles), dim3(kOrderThreads), 0, s, parent, n_nodes,
-                       light_first ? 1 : 0, size, off);
-    hipLaunchKernelGGL(order_finish_kernel, dim3(blocks), dim3(kOrderThreads), 2 * lds_parents, s, parent, n_nodes,
-                       off, perm, rank, status);
+    const int32_t n = (int32_t)n_nodes;
+    int32_t* size = workspace;                 // [n]
+    int32_t* off = size + n;                   // [n]
+    int32_t* kids = off + n;                   // [n + 1]
+    int32_t* first = kids + n + 1;             // [n + 1]
+    int32_t* cursor = first + n + 1;           // [n + 1]
+    int32_t* child = cursor + n + 1;           // [n]
+    const unsigned blocks = (unsigned)((n_nodes + kOrderThreads) / kOrderThreads);   // covers n + 1 entries
+    // (every array is written by a kernel before it is read: nothing of an earlier call survives)
+    hipLaunchKernelGGL(order_init_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, n, size, kids);
+    hipLaunchKernelGGL(order_sizes_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, parent, n, size, kids, status);
+    hipLaunchKernelGGL(order_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, n, kids, first, cursor);
+    hipLaunchKernelGGL(order_fill_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, parent, n, cursor, child);
+    hipLaunchKernelGGL(order_offsets_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, parent, n, light_first ? 1 : 0,
+                       size, kids, first, child, off);
+    hipLaunchKernelGGL(order_finish_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, parent, n, off, perm, rank, status);
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
 }
@@ -321,8 +337,7 @@ extern "C" int fsta_dfs_order(const int64_t* parent, int64_t n_nodes, int32_t li
                               int64_t* rank, int32_t* workspace, uint32_t* status, void* stream) {
     if (n_nodes < 0) return fail(FSTA_EINVAL, "fsta_dfs_order: n_nodes=%lld", (long long)n_nodes);
     if (n_nodes > FSTA_DFS_ORDER_MAX_NODES)
-        return fail(FSTA_EUNSUPPORTED, "fsta_dfs_order: n_nodes=%lld > %d (all-pairs sibling pass)",
-                    (long long)n_nodes, FSTA_DFS_ORDER_MAX_NODES);
+        return fail(FSTA_EUNSUPPORTED, "fsta_dfs_order: n_nodes=%lld > %d", (long long)n_nodes, FSTA_DFS_ORDER_MAX_NODES);
     if (n_nodes == 0) return FSTA_OK;
     if (!parent || !perm || !rank || !workspace || !status)
         return fail(FSTA_EINVAL, "fsta_dfs_order: null pointer");

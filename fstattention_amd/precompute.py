@@ -146,7 +146,7 @@ def dfs_order_gpu(parent: torch.Tensor, children: str = "index", check: bool = T
     n = parent.shape[0]
     perm = torch.empty((n,), dtype=torch.int64, device=dev)
     rank = torch.empty((n,), dtype=torch.int64, device=dev)
-    work = torch.empty((2 * n,), dtype=torch.int32, device=dev)
+    work = torch.empty((_lib.dfs_order_workspace_ints(n),), dtype=torch.int32, device=dev)
     if status is None:
         status = torch.zeros((1,), dtype=torch.int32, device=dev)
     with _on_device(dev):

@@ -252,19 +252,22 @@ int fsta_lineage_from_parents(const int64_t* parent, int64_t n_nodes, int64_t wi
  * lineage and their ancestor lists shrink).  parent[n_nodes] int64 as above ->
  * perm[new_id] = old_id and rank[old_id] = new_id, both int64 [n_nodes].
  * Siblings (and roots) are visited by ascending id, or smallest subtree first
- * (ties by id) when light_first != 0.  workspace: 2 * n_nodes int32 of device
- * scratch.  `status` (zero on entry) gets FSTA_PRE_BAD_NODE_ID for a parent
- * entry outside [-1, i); perm and rank are then the identity.
- * n_nodes <= FSTA_DFS_ORDER_MAX_NODES.
+ * (ties by id) when light_first != 0.  workspace:
+ * FSTA_DFS_ORDER_WORKSPACE_INTS(n_nodes) int32 of device scratch.  `status` (zero
+ * on entry) gets FSTA_PRE_BAD_NODE_ID for a parent entry outside [-1, i); perm
+ * and rank are then the identity.  n_nodes <= FSTA_DFS_ORDER_MAX_NODES (2^17, the
+ * largest entry of the reference's size table, utils.py:4-13).  Work is
+ * O(n_nodes * depth + sum over parents of children^2).
  */
-#define FSTA_DFS_ORDER_MAX_NODES 16384
+#define FSTA_DFS_ORDER_MAX_NODES 131072
+#define FSTA_DFS_ORDER_WORKSPACE_INTS(n) (6 * (size_t)(n) + 8)
 int fsta_dfs_order(const int64_t* parent, int64_t n_nodes, int32_t light_first, int64_t* perm,
                    int64_t* rank, int32_t* workspace, uint32_t* status, void* stream);
 
 /*
  * fsta_dfs_order without a workspace argument and without any allocation: the
- * scratch (2 * n_nodes int32) is an array inside the library, one copy per GPU,
- * held until the process ends (128 KiB).  No counterpart in the reference; for
+ * scratch is an array inside the library, one copy per GPU, held until the
+ * process ends (384 KiB).  No counterpart in the reference; for
  * callers that cannot allocate device memory: code under HIP graph capture,
  * serving loops and harnesses that forbid hipMalloc.  Same arguments, results
  * and status bits as fsta_dfs_order; n_nodes <= FSTA_DFS_ORDER_STATIC_MAX_NODES,

@@ -64,6 +64,9 @@ def test_constants_match_header():
     text = open(HEADER).read()
     defs = dict(re.findall(r"#define\s+(FSTA_[A-Z_0-9]+)\s+(-?\d+)u?\b", text))
     assert int(defs["FSTA_ABI_VERSION"]) == _lib.ABI_VERSION
+    assert int(defs["FSTA_DFS_ORDER_MAX_NODES"]) == _lib.DFS_ORDER_MAX_NODES
+    assert int(defs["FSTA_DFS_ORDER_STATIC_MAX_NODES"]) == _lib.DFS_ORDER_STATIC_MAX_NODES
+    assert "(6 * (size_t)(n) + 8)" in text and _lib.dfs_order_workspace_ints(10) == 68
     assert (int(defs["FSTA_F32"]), int(defs["FSTA_F16"]), int(defs["FSTA_BF16"]), int(defs["FSTA_F64"])) == \
         (_lib.F32, _lib.F16, _lib.BF16, _lib.F64)
     assert int(defs["FSTA_TREE_NOT_PREFIX_CLOSED"]) == _lib.TREE_NOT_PREFIX_CLOSED

@@ -177,7 +177,7 @@ def test_lineage_from_parents_on_gpu():
 @pytest.mark.parametrize("children", ["index", "light_first"])
 def test_dfs_order_on_gpu_matches_the_host_order(children):
     cases = [np.array([-1], dtype=np.int64), np.array([-1, -1, -1], dtype=np.int64)]
-    # up to 4096 nodes one workgroup does everything, beyond that four launches do
+    # up to 4096 nodes one workgroup does everything, beyond that six launches over arrays in device memory do
     for seed, n, window in [(1, 2, None), (2, 300, None), (3, 1500, 8), (4, 2049, 64), (5, 4096, 200),
                             (6, 4097, 16), (7, 9000, None)]:
         parent = trees.random_recursive_parents(n, seed, window)
@@ -199,6 +199,24 @@ def test_dfs_order_on_gpu_matches_the_host_order(children):
         np.testing.assert_array_equal(renumber_parents_gpu(dev_parent, perm, rank).cpu().numpy(), want_parent)
 
 
+@pytest.mark.parametrize("children", ["index", "light_first"])
+def test_dfs_order_on_gpu_at_the_reference_tree_sizes(children):
+    """The reference's benchmark trees go to 2^16 tokens and its size table to 2^17 (utils.py:4-13,
+    fstattention.py:246); plus a wide star, a deep chain and a large random forest."""
+    cases = [trees.parents_from_lineage(*(t.numpy() for t in trees.create_tree(depth))) for depth in (13, 14)]
+    cases.append(trees.random_recursive_parents(100000, 21, 500))
+    cases[-1][::977] = -1
+    star = np.zeros(20000, dtype=np.int64)
+    star[0] = -1
+    cases.append(star)
+    cases.append(np.arange(-1, 29999, dtype=np.int64))          # a chain of 30000 levels
+    for parent in cases:
+        want = trees.dfs_order(parent, children)
+        perm, rank = dfs_order_gpu(torch.from_numpy(parent).cuda(), children)
+        np.testing.assert_array_equal(perm.cpu().numpy(), want)
+        np.testing.assert_array_equal(rank.cpu().numpy()[want], np.arange(len(parent)))
+
+
 def test_dfs_order_on_gpu_flags_bad_parents_and_sizes():
     with pytest.raises(ValueError):
         dfs_order_gpu(torch.tensor([-1, 0, 5, 1], dtype=torch.int64).cuda())
@@ -207,7 +225,11 @@ def test_dfs_order_on_gpu_flags_bad_parents_and_sizes():
     perm, rank = dfs_order_gpu(torch.tensor([-1, -3, 0], dtype=torch.int64).cuda(), check=False)
     assert perm.tolist() == [0, 1, 2] and rank.tolist() == [0, 1, 2]   # identity when flagged
     with pytest.raises(RuntimeError):
-        dfs_order_gpu(torch.full((16385,), -1, dtype=torch.int64).cuda())
+        dfs_order_gpu(torch.full((131073,), -1, dtype=torch.int64).cuda())
+    big = torch.from_numpy(trees.random_recursive_parents(50000, 3, 100)).cuda()
+    big[40000] = 45000
+    perm, rank = dfs_order_gpu(big, check=False)
+    assert torch.equal(perm, torch.arange(50000, device="cuda")) and torch.equal(rank, perm)
     empty, _ = dfs_order_gpu(torch.empty((0,), dtype=torch.int64).cuda())
     assert empty.numel() == 0
 

@@ -36,7 +36,7 @@ def test_static_scratch_entry_point_matches_the_workspace_one():
     for n, seed, window, light in ((12000, 5, 64, 1), (5000, 6, None, 0), (limit, 7, 8, 1), (4097, 8, 200, 0), (300, 9, 16, 1)):
         host_parent = trees.random_recursive_parents(n, seed, window)
         parent = torch.from_numpy(host_parent).cuda()
-        work = torch.full((2 * n,), 0x5A5A5A5A, dtype=torch.int32, device="cuda")
+        work = torch.full((_lib.dfs_order_workspace_ints(n),), 0x5A5A5A5A, dtype=torch.int32, device="cuda")
         want = _order(lib, "workspace", parent, light, work)
         got = _order(lib, "static", parent, light, None)
         assert got[2] == 0 and want[2] == 0
