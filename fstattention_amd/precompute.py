@@ -14,6 +14,9 @@ from . import _lib
 from .attention import PackedTreeMask, _cache_key, _on_device, _stream_ptr
 
 
+MEDUSA_MAX_CANDIDATES = 16384      # candidate paths fsta_medusa_tree ranks in one launch
+
+
 def _raise_for_status(status: int, max_ancestors: int):
     if status & _lib.PRE_BAD_NODE_ID:
         raise ValueError("lineage holds a node id outside [-1, n_nodes)")
@@ -180,8 +183,8 @@ def medusa_parents_gpu(probs: torch.Tensor, n: int, check: bool = False, status=
     ``n-1`` best paths are kept (ties: shallower first, then smaller ranks) and numbered by
     ``(depth, ranks)``; node 0 is the empty path.  Scores are formed in float64 in the host
     version's multiplication order.  One launch of a HIP kernel on the current stream
-    (``fsta_medusa_tree``; up to 16384 candidate paths, beyond that the same steps run as torch
-    tensor operations); with ``dfs_order_gpu``, ``lineage_from_parents_gpu(width=depths + 1)`` and
+    (``fsta_medusa_tree``; up to 16384 candidate paths = sum of ``topk**d``, e.g. four heads of 10
+    ranks or three of 24; more are refused); with ``dfs_order_gpu``, ``lineage_from_parents_gpu(width=depths + 1)`` and
     ``create_fst_attention_kernel_inputs(check=False)`` a tree goes from draft-head probabilities
     to kernel inputs without touching the host.  ``check`` synchronises and raises when a kept
     path's prefix was not kept (probabilities above 1 or not numbers).  ``status``: optional zeroed
@@ -193,8 +196,10 @@ def medusa_parents_gpu(probs: torch.Tensor, n: int, check: bool = False, status=
     total = sum(topk ** d for d in range(1, depths + 1))
     if not 1 <= n <= total + 1:
         raise ValueError(f"n={n} outside [1, {total + 1}] for depths={depths}, topk={topk}")
-    if total > 16384 or depths * topk > 1024:
-        return _medusa_parents_torch(probs, n)
+    if total > MEDUSA_MAX_CANDIDATES or depths * topk > 1024:
+        raise ValueError(f"depths={depths}, topk={topk} give {total} candidate paths; the tree builder takes at most "
+                         f"{MEDUSA_MAX_CANDIDATES} (the scores of all candidates live in one workgroup's LDS) and "
+                         f"depths * topk <= 1024")
     if probs.dtype not in (torch.float32, torch.float64):
         probs = probs.to(torch.float64)
     probs = probs.contiguous()
@@ -209,28 +214,3 @@ def medusa_parents_gpu(probs: torch.Tensor, n: int, check: bool = False, status=
     if check and int(status.item()) & _lib.TREE_NOT_PREFIX_CLOSED:
         raise ValueError("the kept paths are not closed under prefixes (probabilities above 1 or not numbers)")
     return parent
-
-
-def _medusa_parents_torch(probs: torch.Tensor, n: int) -> torch.Tensor:
-    """The steps of ``fsta_medusa_tree`` as torch tensor operations (any number of candidate paths)."""
-    depths, topk = probs.shape
-    probs = probs.to(torch.float64)
-    dev = probs.device
-    # all paths in (depth, ranks) order: level d is the outer product of level d-1 with probs[d-1]
-    levels, score = [], torch.ones((1,), dtype=torch.float64, device=dev)
-    for d in range(depths):
-        score = (score[:, None] * probs[d][None, :]).reshape(-1)
-        levels.append(score)
-    scores = torch.cat(levels)                                   # key k -> path k + 1 in that order
-    best = torch.sort(scores, descending=True, stable=True).indices[: n - 1]   # stable: ties keep key order
-    kept = torch.sort(best).values + 1                           # keys of nodes 1 .. n-1 (key 0 = root)
-    # key -> (depth, value): value = ranks read as a base-topk number; the parent drops the last digit
-    starts = [1]
-    for d in range(1, depths + 1):
-        starts.append(starts[-1] + topk ** d)
-    bounds = torch.tensor(starts, dtype=torch.int64, device=dev)
-    level = torch.bucketize(kept, bounds, right=True) - 1        # 0-based depth index (depth - 1)
-    value = kept - bounds[level]
-    parent_key = torch.where(level > 0, bounds[(level - 1).clamp(min=0)] + value // topk, torch.zeros_like(kept))
-    parent_id = torch.where(parent_key > 0, torch.searchsorted(kept, parent_key) + 1, torch.zeros_like(kept))
-    return torch.cat([torch.full((1,), -1, dtype=torch.int64, device=dev), parent_id])

@@ -260,9 +260,9 @@ def test_medusa_tree_built_on_the_gpu_matches_the_host_builder():
     big = trees.medusa_probs(4, 11, 0.3, 12)       # 16104 candidate paths: the largest the kernel takes
     np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(big).cuda(), 1000).cpu().numpy(),
                                   trees.medusa_parents_from_probs(big, 1000))
-    wide = trees.medusa_probs(2, 200, 0.3, 13)     # 40200 paths: tensor operations instead of the kernel
-    np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(wide).cuda(), 300).cpu().numpy(),
-                                  trees.medusa_parents_from_probs(wide, 300))
+    wide = trees.medusa_probs(2, 200, 0.3, 13)     # 40200 paths: more than one launch ranks, refused
+    with pytest.raises(ValueError, match="candidate paths"):
+        medusa_parents_gpu(torch.from_numpy(wide).cuda(), 300)
     with pytest.raises(ValueError):                # a deeper path scoring above its prefix
         medusa_parents_gpu(torch.tensor([[0.5, 0.1], [3.0, 0.1]], dtype=torch.float64).cuda(), 2, check=True)
 
