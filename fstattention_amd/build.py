@@ -79,22 +79,30 @@ def _split_resource_remarks(stderr: str):
     return usage, "\n".join(rest)
 
 
-def build_library(verbose: bool = True, jobs: int | None = None) -> str:
-    """Compiles every source and links ``libfsta.so``; always rebuilds."""
+TIMELINE_LIB_PATH = os.path.join(PKG_DIR, "libfsta_timeline.so")
+
+
+def build_library(verbose: bool = True, jobs: int | None = None, timeline: bool = False) -> str:
+    """Compiles every source and links ``libfsta.so``; always rebuilds.  ``timeline=True`` builds the
+    instrumented variant ``libfsta_timeline.so`` instead (``-DFSTA_TIMELINE``: the matrix-core kernel notes
+    cycle stamps, see ``fstattention_amd/timeline.py``); the regular library is left alone."""
     hipcc = _hipcc()
-    os.makedirs(OBJ_DIR, exist_ok=True)
+    obj_dir = OBJ_DIR + ("_timeline" if timeline else "")
+    lib_path = TIMELINE_LIB_PATH if timeline else LIB_PATH
+    extra = ["-DFSTA_TIMELINE"] if timeline else []
+    os.makedirs(obj_dir, exist_ok=True)
     jobs = jobs or min(len(SOURCES), os.cpu_count() or 1, 16)
 
     def compile_one(src):
-        obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
-        warn = _run([hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj])
+        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
+        warn = _run([hipcc, *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj])
         return obj, warn
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         results = list(pool.map(compile_one, SOURCES))
     for (obj, warn), src in zip(results, SOURCES):
         usage, warn = _split_resource_remarks(warn)
-        if src in NO_SCRATCH:
+        if src in NO_SCRATCH and not timeline:
             bad = [(name, u) for name, u in usage.items() if u.get("ScratchSize [bytes/lane]", 0)]
             if bad:
                 raise RuntimeError(f"{src}: kernels using scratch memory: " +
@@ -104,12 +112,12 @@ def build_library(verbose: bool = True, jobs: int | None = None) -> str:
         if verbose and warn.strip():
             sys.stderr.write(warn + "\n")
     objs = [o for o, _ in results]
-    tmp = LIB_PATH + ".tmp"
+    tmp = lib_path + ".tmp"
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs])
-    os.replace(tmp, LIB_PATH)
+    os.replace(tmp, lib_path)
     if verbose:
-        print(f"built {LIB_PATH} ({os.path.getsize(LIB_PATH)} bytes)")
-    return LIB_PATH
+        print(f"built {lib_path} ({os.path.getsize(lib_path)} bytes)")
+    return lib_path
 
 
 TORCH_OPS_PATH = os.path.join(PKG_DIR, "_fsta_torch.so")
@@ -138,5 +146,8 @@ def build_torch_ops(verbose: bool = True) -> str:
 
 
 if __name__ == "__main__":
-    build_library()
-    build_torch_ops()
+    if "--timeline" in sys.argv[1:]:
+        build_library(timeline=True)
+    else:
+        build_library()
+        build_torch_ops()

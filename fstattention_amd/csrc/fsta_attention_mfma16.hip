@@ -20,6 +20,22 @@ namespace {
 
 using namespace mfma;
 
+// Instrumented build (-DFSTA_TIMELINE, `python -m fstattention_amd.build --timeline`): every wave
+// notes the 100 MHz clock at fixed points of the kernel and writes the notes out at the end;
+// `python -m fstattention_amd.timeline` turns them into the mean time between the points.  The
+// regular library contains none of this.
+#ifdef FSTA_TIMELINE
+constexpr int kStamps = 16;
+__device__ uint64_t* g_timeline = nullptr;     // [workgroup][wave][kStamps + 2], set by fsta_timeline_buffer
+__device__ __forceinline__ uint32_t stamp_clock() {
+    // the constant 100 MHz clock (10 ns per tick, the same on every CU)
+    return (uint32_t)__builtin_amdgcn_s_memrealtime();
+}
+#define FSTA_STAMP(i) do { if (lane == 0) tl_s[wave][i] = stamp_clock(); } while (0)
+#else
+#define FSTA_STAMP(i) do { } while (0)
+#endif
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
@@ -170,6 +186,12 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+#ifdef FSTA_TIMELINE
+    __shared__ uint32_t tl_s[16][kStamps];
+    const uint64_t tl_begin = __builtin_amdgcn_s_memrealtime();     // 100 MHz, the same clock on every CU
+    if ((tid & 63) < kStamps) tl_s[wave][tid & 63] = 0u;
+    { const int lane = tid & 63; FSTA_STAMP(0); }
+#endif
     const int qgroup = wave % kQGroups;   // which 16 query rows
     const int split = wave / kQGroups;    // which share of the tiles (of the head dimension)
     const int dt0 = kDShare ? split * kOTiles : 0;   // first accumulator tile of this wave
@@ -302,6 +324,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         issue_rows(t, t, rows);
     }
 
+    FSTA_STAMP(1);    // all start-up requests are out
     const bool gathers = !(kDmaWaves < kWaves && wave >= kDmaWaves);
     // Q fragments: B operand of S^T = K.Q^T, lane holds Q[q][32s + 8g .. +7].  Only the leaf
     // tiles requested above were issued after the Q rows.
@@ -327,6 +350,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         read_q(0);        // Q sits in ring slots the gathers are about to take (waits for all of this wave's transfers)
         ring_barrier();   // everybody's pieces of the plan have landed, everybody has read its Q rows
     }
+    FSTA_STAMP(2);    // the plan is here
     // From the plan: ancestor count, validity of this lane's own leaf slot and, after early leaf
     // requests, whether any valid leaf slot names another row than the one requested (lane i looks
     // at slot i of the tiles requested: every wave sees all of them and decides alike).
@@ -508,7 +532,9 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         issue_slot = 0;
     }
     refill();
+    FSTA_STAMP(3);    // ancestor tiles requested
     if (early_leaf) read_q(issued);
+    FSTA_STAMP(4);    // Q fragments in registers
 
     float m_i = -INFINITY, l_i = 0.f;
     f32x4 o[kOTiles];
@@ -520,6 +546,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     // per query from it on the vector ALU and seed their running softmax with it.
     for (int base = tree ? 0 : kLeafTiles; base < kLeafTiles; base += kLeafGroup) {
         begin_step(kLeafGroup);
+        FSTA_STAMP(5);    // (last) leaf tile has landed
         const int my_tile = qgroup >> 1;
         if ((kDShare || split == 0) && my_tile >= base && my_tile < base + kLeafGroup && __ballot(leaf_ok) != 0ull) {
             const T* kt = tile_ptr(my_tile - base);
@@ -565,6 +592,10 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         }
         end_step(kLeafGroup);
     }
+    FSTA_STAMP(6);    // leaf step done
+#ifdef FSTA_TIMELINE
+    int tl_tile = 0;
+#endif
 
     // Ancestor tiles under the packed tree mask, then the dense shared prefix; kSplit tiles per
     // step, tile consumed+s by the waves of share s.
@@ -579,6 +610,10 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     // this row's mask words, one per ancestor tile (bits of empty slots are clear in the plan)
     const uint32_t* my_mask = group_s + (row_in_block >> 5) * group_words + kTileN + (row_in_block & 31);
     while (consumed < total_tiles) {
+#ifdef FSTA_TIMELINE
+        if (tl_tile < 5) { FSTA_STAMP(7 + tl_tile); }     // begin of ancestor / prefix step tl_tile
+        ++tl_tile;
+#endif
         begin_step(kSplit);
         const int t = consumed + (kDShare ? 0 : split);
         const T* kt = tile_ptr(kDShare ? 0 : split);
@@ -712,6 +747,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         }
     }
 
+    FSTA_STAMP(12);   // all tiles done
     // ---- end of the tile list: normalise, write O once (and the base-2 log-sum-exp) --------
     // In the accumulator layout 16 neighbouring lanes hold 16 different rows of O, which the
     // memory pipeline would write as 64 separate 8-byte pieces per instruction.  A wave turns
@@ -770,6 +806,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     };
     if constexpr (kDShare) {
         __syncthreads();   // every wave is done with the last tile
+        FSTA_STAMP(15);   // (head-dimension pairing) barrier in front of the epilogue passed
         finish(o, split * (D / 2), smem + (size_t)wave * 16 * kStageStride, split == 0);
     } else if constexpr (kSplit == 1) {
         __syncthreads();   // every wave is done with the last tile
@@ -815,6 +852,16 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         unsigned char* stage = smem + (size_t)kQGroups * 2 * kXchFloats * 4 + (size_t)wave * 16 * kStageStride;
         finish(keep, split * (D / 2), stage, split == 0);
     }
+#ifdef FSTA_TIMELINE
+    FSTA_STAMP(13);   // stores issued
+    wait_vmcnt<0>();
+    FSTA_STAMP(14);   // stores retired
+    if (g_timeline && lane < kStamps + 2) {
+        const uint64_t wg = (uint64_t)blockIdx.x + (uint64_t)gridDim.x * (blockIdx.y + (uint64_t)gridDim.y * blockIdx.z);
+        uint64_t* out = g_timeline + (wg * kWaves + wave) * (kStamps + 2);
+        out[lane] = lane < kStamps ? tl_s[wave][lane] : lane == kStamps ? tl_begin : __builtin_amdgcn_s_memrealtime();
+    }
+#endif
 }
 
 template <bool BF16, int D, int M, bool SPLIT, int KS>
@@ -981,3 +1028,12 @@ int launch_attention_mfma16(const AttnParams& p, int dtype, int head_dim, bool f
 }
 
 }  // namespace fsta
+
+#ifdef FSTA_TIMELINE
+// Instrumented build only: device buffer of (workgroups x waves x 18) uint64 that every launch of
+// the kernel above fills (16 stamps of the 100 MHz clock, then the full clock at entry and exit), or NULL.
+extern "C" int fsta_timeline_buffer(uint64_t* device_buffer) {
+    FSTA_HIP_OK(hipMemcpyToSymbol(HIP_SYMBOL(fsta::g_timeline), &device_buffer, sizeof(device_buffer)));
+    return FSTA_OK;
+}
+#endif

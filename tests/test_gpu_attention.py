@@ -121,6 +121,27 @@ def test_config5_full_size_sampled_rows(order):
     torch.testing.assert_close(o[7:, 63:], one, atol=2e-3, rtol=2e-3)
 
 
+def test_config5_layer_loop_shares_one_set_of_kernel_inputs():
+    """Configuration 5 as it is timed: the kernel inputs are built ONCE on the GPU from the device-resident
+    parent array and reused by every layer, each layer with fresh seeded q/k/v (seed = tensor seed + layer).
+    Three of the 32 layers, all 8 x 64 slices each, sampled rows against the host."""
+    cfg = trees.config(5)
+    m, d, n = cfg.block_m, cfg.head_dim, cfg.n_nodes
+    max_anc = trees.required_max_ancestors(cfg.parent, m, 16)
+    parent_dev = torch.from_numpy(cfg.parent).cuda()
+    lineage, level = lineage_from_parents_gpu(parent_dev)
+    a_idx, packed, l_idx = create_fst_attention_kernel_inputs(lineage, level, m, max_anc, want_bool_mask=False)
+    scale = 1.0 / math.sqrt(d)
+    for layer in (0, 13, cfg.layers - 1):
+        g = torch.Generator(device="cuda").manual_seed(cfg.tensor_seed + layer)
+        q, k, v = (torch.randn((cfg.batch, cfg.heads, n, d), generator=g, device="cuda", dtype=torch.float32)
+                   .to(torch.bfloat16) for _ in range(3))
+        o, lse = fst_attention(q, k, v, a_idx, packed, l_idx, scale, BLOCK_M=m, MAX_ANCESTORS=max_anc,
+                               out_dtype=torch.float32, return_lse=True)
+        sampled_rows_check(q, k, v, cfg.parent, o, lse, scale, 0, 48, 100 + layer, torch.bfloat16, f"cfg5 layer {layer}")
+        del q, k, v, o
+
+
 def test_large_tree_behind_a_long_prefix_sampled_rows():
     """40000 tokens behind 5000 prefix keys, 3 heads: index arithmetic far beyond the benchmark sizes
     (key runs chosen by the library), checked on sampled rows."""
