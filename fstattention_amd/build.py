@@ -27,6 +27,7 @@ SOURCES = [
     "fsta_attention_generic.hip",
     "fsta_attention_mfma.hip",
     "fsta_attention_mfma16.hip",
+    "fsta_attention_prefix.hip",
 ]
 
 # packed-fp32 VALU forms are switched off for device code on purpose
@@ -39,7 +40,7 @@ HIPCC_FLAGS = [
 
 # Kernels of these sources must keep everything in registers: a private array the compiler leaves
 # in scratch memory, or a spill, is reloaded through the same vmcnt queue their gather rings count on.
-NO_SCRATCH = ("fsta_attention_mfma16.hip", "fsta_attention_mfma.hip")
+NO_SCRATCH = ("fsta_attention_mfma16.hip", "fsta_attention_mfma.hip", "fsta_attention_prefix.hip")
 
 
 def _hipcc() -> str:

@@ -36,23 +36,7 @@ __device__ __forceinline__ uint32_t stamp_clock() {
 #define FSTA_STAMP(i) do { } while (0)
 #endif
 
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
-}
-__device__ __forceinline__ f32x4 mfma16(f16x8 a, f16x8 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
-}
-
 constexpr int leaf_group16_for(int block_m) { return block_m >= 64 ? 2 : 1; }
-
-// V tile swizzle for the transposing read of this kernel: one read instruction touches 16
-// consecutive rows x 32 bytes, so 32-byte granules are XORed with the row.
-template <int D> __device__ __forceinline__ int v16_chunk(int row, int c) {
-    constexpr int gpr = D / 16, rpb = 8 / gpr;   // granules per row, rows per 256 bytes
-    return c ^ (2 * ((row / rpb) % gpr));
-}
 
 // LDS of one workgroup: the ring of K|V tiles, then the workgroup's part of the block plan
 // (header and ancestor keys, then leaf keys and mask words of its M/32 groups of 32 rows).
@@ -87,7 +71,9 @@ __device__ __forceinline__ void flush_rows(const unsigned char* stage, int strid
 // and stores its half of O.  Nothing is exchanged or merged at the end, which shortens the chain
 // of a launch with one or two ancestor tiles per block; the duplicated S and softmax work makes
 // it the wrong choice for long tile lists.
-// RUNS = the launch cuts the shared prefix into runs of keys (AttnParams::key_splits > 1).
+// RUNS = the launch writes partial results into a workspace (AttnParams::part_o): workgroup `ksp` of a block
+// takes the ksp-th run of prefix tiles (key_splits runs of split_tiles tiles; none at all with split_tiles = 0,
+// when the prefix is another kernel's), workgroup 0 also the tree part.
 // KV8 = K and V are stored as 8-bit floats (OCP e4m3) with one scale per (batch, head) slice each:
 // rows are gathered as they are (half the bytes) into a staging ring; the workgroup widens every
 // tile once into one of two 16-bit tiles in LDS (exact: e4m3 is a subset of both 16-bit types),
@@ -876,7 +862,7 @@ int launch_ks(const AttnParams& p, int sub_shift, hipStream_t stream) {
     constexpr int kShares = KS < 0 ? -KS : KS;
     constexpr int kWaves = M / 16 * kShares, kQSlots = (kWaves * 16 + 2 * kTileN - 1) / (2 * kTileN);
     if (stages < kQSlots + (M / 32 < 2 ? M / 32 : 2)) {
-        if (p.key_splits > 1) return FSTA_EUNSUPPORTED;   // the caller falls back to a launch without key splits
+        if (p.part_o) return FSTA_EUNSUPPORTED;   // the caller falls back to a launch without key splits
         return launch_attention_mfma(p, BF16 ? FSTA_BF16 : FSTA_F16, D, BF16 && !SPLIT, stream);
     }
     // the epilogue reuses the front of the segment: exchange area of a key split, row staging
@@ -894,9 +880,9 @@ int launch_ks(const AttnParams& p, int sub_shift, hipStream_t stream) {
     const int shift_arg = sub_shift | (linear_grid ? 0x100 : 0);
     // a launch whose workgroups all run at once: leaf tiles requested early, Q in an area of its own
     constexpr size_t kQBytes = (size_t)kWaves * 16 * D * 2;
-    const int early = grid <= kCus && p.key_splits == 1 && lds + kQBytes <= 160 * 1024 ? 1 : 0;
+    const int early = grid <= kCus && !p.part_o && lds + kQBytes <= 160 * 1024 ? 1 : 0;
     if (early) lds += kQBytes;
-    if (p.key_splits > 1) {
+    if (p.part_o) {
         if constexpr (KS > 0) {
             if (lds > 64 * 1024) {
                 const int rc = allow_full_lds<&attn_mfma16_kernel<BF16, D, M, SPLIT, KS, true>>();
@@ -916,7 +902,7 @@ int launch_ks(const AttnParams& p, int sub_shift, hipStream_t stream) {
                            stream, p, stages, early, shift_arg);
     }
     FSTA_HIP_OK(hipGetLastError());
-    note_launch({"attn_mfma16_kernel", BF16 ? "true" : "false", {D, M, SPLIT ? 1 : 0, KS, p.key_splits > 1 ? 1 : 0, 0}, 6,
+    note_launch({"attn_mfma16_kernel", BF16 ? "true" : "false", {D, M, SPLIT ? 1 : 0, KS, p.part_o ? 1 : 0, 0}, 6,
                  0x34u, sub_shift, early});
     return FSTA_OK;
 }
@@ -935,7 +921,7 @@ int launch_one(const AttnParams& p, int sub_shift, hipStream_t stream) {
             // and so it does with longer lists (8 tiles: +10 %).
             const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
             const bool one_round = kXcds * slices_per_xcd * (p.nb << sub_shift) <= kCus;
-            if (one_round && work_tiles <= 4 && p.prefix == 0 && p.key_splits == 1 && !p.share_tiles)
+            if (one_round && work_tiles <= 4 && p.prefix == 0 && !p.part_o && !p.share_tiles)
                 return launch_ks<BF16, D, M, SPLIT, -2>(p, sub_shift, stream);
         }
         if (work_tiles >= 2) return launch_ks<BF16, D, M, SPLIT, 2>(p, sub_shift, stream);
@@ -947,7 +933,7 @@ template <bool BF16, int D, bool SPLIT>
 int launch_m(const AttnParams& p, hipStream_t stream) {
     // Launches that would leave half of the CUs without a workgroup are cut into half-blocks.
     const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
-    const bool halve = kXcds * slices_per_xcd * p.nb * 2 * p.key_splits <= kCus;
+    const bool halve = !p.part_o && kXcds * slices_per_xcd * p.nb * 2 <= kCus;
     switch (p.block_m) {
         case 32: return launch_one<BF16, D, 32, SPLIT>(p, 0, stream);
         case 64: return halve ? launch_one<BF16, D, 32, SPLIT>(p, 1, stream) : launch_one<BF16, D, 64, SPLIT>(p, 0, stream);

@@ -78,6 +78,35 @@ size_t key_split_bytes(int splits, int64_t slices, int nq, int head_dim) {
     return (size_t)splits * (size_t)slices * (size_t)nq * (size_t)(head_dim + 1) * sizeof(float);
 }
 
+constexpr int kDenseMinKeys = 2048;   // shortest prefix handed to the dense prefix kernel (below: two more launches cost more than they save)
+constexpr int kDenseRows = 128;       // query rows per workgroup of that kernel
+
+// Whether (and how) the prefix goes to the dense prefix kernel: number of key runs (0 = not at all) and
+// prefix tiles per run.  The tree part then takes one more workspace slot.  Shape and flags only.
+int plan_dense_prefix(int64_t slices, int nq, int nk, int head_dim, int dtype, int block_m, float sm_scale,
+                      uint32_t flags, int* split_tiles) {
+    const int prefix = nk - nq;
+    if (slices <= 0 || nq <= 0 || prefix < kDenseMinKeys) return 0;
+    if ((flags & (FSTA_FLAG_GENERIC | FSTA_FLAG_WIDE_WAVES)) || !(sm_scale > 0.f) ||
+        !mfma_supported(dtype, head_dim, block_m) || !prefix_kernel_supported(dtype, head_dim))
+        return 0;
+    const int forced = (int)((flags >> 8) & 0xffu);
+    if (forced == 1) return 0;        // "never split": the prefix stays in the tree kernel's own loop
+    const int tiles = (prefix + kKeyTile - 1) / kKeyTile;
+    int64_t want = forced;
+    if (!forced) {
+        const int64_t groups = ((slices + 7) / 8) * 8 * ((nq + kDenseRows - 1) / kDenseRows);
+        want = (kTargetGroups + groups - 1) / groups;
+        if (want > tiles / kMinRunTiles) want = tiles / kMinRunTiles;
+        if (want < 1) want = 1;
+    }
+    if (want > tiles) want = tiles;
+    if (want > 254) want = 254;
+    const int per = (int)((tiles + want - 1) / want);
+    *split_tiles = per;
+    return (tiles + per - 1) / per;
+}
+
 }  // namespace
 
 extern "C" size_t fsta_attention_workspace_bytes(int32_t batch, int32_t heads, int32_t nq, int32_t nk,
@@ -87,6 +116,8 @@ extern "C" size_t fsta_attention_workspace_bytes(int32_t batch, int32_t heads, i
     if (batch <= 0 || heads <= 0 || nq <= 0 || nk <= nq || block_m <= 0) return 0;
     int split_tiles = 0;
     const int64_t slices = (int64_t)batch * heads;
+    const int runs = plan_dense_prefix(slices, nq, nk, head_dim, dtype, block_m, sm_scale, flags, &split_tiles);
+    if (runs > 0) return key_split_bytes(runs + 1, slices, nq, head_dim);
     const int splits = plan_key_splits(slices, nq, nk, head_dim, dtype, block_m, sm_scale, flags, &split_tiles);
     return splits > 1 ? key_split_bytes(splits, slices, nq, head_dim) : 0;
 }
@@ -167,8 +198,33 @@ extern "C" int fsta_attention_fwd_ws(const void* q, const void* k, const void* v
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (workspace && p.plan) {
+        // a long prefix goes to the dense prefix kernel, run by run; the tree kernel does the tree part only
+        // (slot 0 of the workspace) and one merge joins everything
+        int run_tiles = 0;
+        const int runs = plan_dense_prefix(slices, nq, nk, head_dim, dtype, block_m, sm_scale, flags, &run_tiles);
+        if (runs > 0 && workspace_bytes >= key_split_bytes(runs + 1, slices, nq, head_dim)) {
+            if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+                return fail(FSTA_EINVAL, "fsta_attention_fwd_ws: workspace must be 16-byte aligned");
+            const bool fast_pv = (flags & FSTA_FLAG_FAST_PV) != 0;
+            AttnParams pt = p;
+            pt.part_o = static_cast<float*>(workspace);
+            pt.part_lse = pt.part_o + (size_t)(runs + 1) * slices * nq * head_dim;
+            pt.key_splits = 1;
+            pt.split_tiles = 0;        // no prefix tile for the tree kernel
+            int rc = launch_attention_mfma16(pt, dtype, head_dim, fast_pv, s);
+            if (rc == FSTA_OK) {
+                pt.key_splits = runs;
+                pt.split_tiles = run_tiles;
+                rc = launch_attention_prefix(pt, dtype, head_dim, fast_pv, s);
+                if (rc != FSTA_OK) return rc;
+                return launch_merge_splits(pt.part_o, pt.part_lse, runs + 1, slices * nq, head_dim, o, out_dtype, lse, s);
+            }
+            if (rc != FSTA_EUNSUPPORTED) return rc;
+            // (ancestor lists too long for the kernel with key runs: the launches below)
+        }
         int split_tiles = 0;
-        const int splits = plan_key_splits(slices, nq, nk, head_dim, dtype, block_m, sm_scale, flags, &split_tiles);
+        // (a workspace too small for what fsta_attention_workspace_bytes asked for: no split of any kind)
+        const int splits = runs > 0 ? 1 : plan_key_splits(slices, nq, nk, head_dim, dtype, block_m, sm_scale, flags, &split_tiles);
         if (splits > 1 && workspace_bytes >= key_split_bytes(splits, slices, nq, head_dim)) {
             if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
                 return fail(FSTA_EINVAL, "fsta_attention_fwd_ws: workspace must be 16-byte aligned");

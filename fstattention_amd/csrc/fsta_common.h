@@ -112,6 +112,9 @@ int launch_attention_mfma(const AttnParams& p, int dtype, int head_dim, bool fas
                           hipStream_t stream);
 int launch_attention_mfma16(const AttnParams& p, int dtype, int head_dim, bool fast_pv,
                             hipStream_t stream);
+// dense shared prefix, run by run, into slots 1 .. key_splits of p.part_o / p.part_lse
+int launch_attention_prefix(const AttnParams& p, int dtype, int head_dim, bool fast_pv, hipStream_t stream);
+bool prefix_kernel_supported(int dtype, int head_dim);
 int launch_attention_mfma16_kv8(const AttnParams& p, int dtype, int head_dim, hipStream_t stream);
 bool mfma_supported(int dtype, int head_dim, int block_m);
 // joins `splits` partial results (layout of AttnParams::part_o / part_lse) into o (and lse, may be null)

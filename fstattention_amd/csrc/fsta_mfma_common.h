@@ -215,5 +215,21 @@ template <int D> __device__ __forceinline__ int v_chunk(int row, int c) {
     return c ^ (4 * ((row / rpb) % qpr));
 }
 
+// V tile swizzle for the transposing read of the kernels with 16 query rows per MFMA: one read
+// instruction touches 16 consecutive rows x 32 bytes, so 32-byte granules are XORed with the row.
+template <int D> __device__ __forceinline__ int v16_chunk(int row, int c) {
+    constexpr int gpr = D / 16, rpb = 8 / gpr;   // granules per row, rows per 256 bytes
+    return c ^ (2 * ((row / rpb) % gpr));
+}
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mfma16(f16x8 a, f16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
 }  // namespace mfma
 }  // namespace fsta

@@ -157,13 +157,20 @@ def test_workspace_planning_is_host_arithmetic():
     lib = _lib.load()
     per_run = 32 * 256 * (128 + 1) * 4       # float32 partial rows + their log-sum-exps of one run
     size = lambda *a: lib.fsta_attention_workspace_bytes(*a)
-    # one sequence, 32 heads, 4 blocks of 64 rows behind 16384 prefix keys: 128 workgroups -> 4 runs
-    assert size(1, 32, 256, 256 + 16384, 128, _lib.BF16, 64, 64, 0.1, 0) == 4 * per_run
-    assert size(1, 32, 256, 256 + 16384, 128, _lib.BF16, 64, 64, 0.1, _lib.flag_key_splits(7)) == 7 * per_run
+    # one sequence, 32 heads, 256 rows behind 16384 prefix keys: the prefix goes to the dense prefix kernel, 64 workgroups
+    # of 128 rows per run -> 8 runs, plus one slot for the tree part
+    assert size(1, 32, 256, 256 + 16384, 128, _lib.BF16, 64, 64, 0.1, 0) == 9 * per_run
+    assert size(1, 32, 256, 256 + 16384, 128, _lib.BF16, 64, 64, 0.1, _lib.flag_key_splits(7)) == 8 * per_run
+    # enough workgroups to begin with: one run (the dense kernel still takes the prefix)
+    assert size(8, 32, 256, 256 + 16384, 128, _lib.BF16, 64, 64, 0.1, 0) == 2 * 8 * per_run
+    # head dims the dense kernel does not take: runs of keys inside the tree kernel (4 for 128 workgroups)
+    assert size(1, 32, 256, 256 + 16384, 32, _lib.BF16, 64, 64, 0.1, 0) == 4 * 32 * 256 * (32 + 1) * 4
     # nothing to cut: no prefix, a short one, enough blocks already, never-split flag
     assert size(1, 32, 256, 256, 128, _lib.BF16, 64, 64, 0.1, 0) == 0
     assert size(1, 32, 256, 256 + 256, 128, _lib.BF16, 64, 64, 0.1, 0) == 0
-    assert size(8, 32, 256, 256 + 16384, 128, _lib.BF16, 64, 64, 0.1, 0) == 0
+    # a prefix too short for the dense kernel: runs of keys inside the tree kernel
+    assert size(1, 32, 256, 256 + 1024, 128, _lib.BF16, 64, 64, 0.1, 0) == 4 * per_run
+    assert size(8, 32, 256, 256 + 16384, 32, _lib.BF16, 64, 64, 0.1, 0) == 0
     assert size(1, 32, 256, 256 + 16384, 128, _lib.BF16, 64, 64, 0.1, _lib.flag_key_splits(1)) == 0
     # kernels without key runs: float32, the scalar and wide-wave kernels, non-positive scales
     assert size(1, 32, 256, 256 + 16384, 128, _lib.F32, 64, 64, 0.1, 0) == 0

@@ -224,6 +224,17 @@ def test_prefix_cut_into_key_runs(dtype, block_m, d, prefix, splits):
     run_tree(parent, block_m, 1, 3, d, dtype, 13, prefix=prefix, key_splits=splits)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("scale", [0.3, 1.0])
+def test_dense_prefix_kernel_with_peaked_weights(dtype, scale):
+    """A long prefix goes to the dense prefix kernel, which feeds bfloat16 weights to the matrix cores as single
+    values.  Scores scaled up until one or two keys carry nearly all the weight of a row: the rounding of single
+    weights must still stay inside the tolerance (2e-3 on the float32 output)."""
+    parent = trees.random_recursive_parents(256, 77, window=32)
+    run_tree(parent, 64, 1, 4, 128, dtype, 23, prefix=4096, scale=scale)
+    run_tree(parent, 128, 2, 2, 64, dtype, 24, prefix=2048, scale=scale)
+
+
 def test_key_runs_native_output_type_and_workspace_contract():
     """Output in the storage type through the joining kernel; the C entry point with no or too
     small a workspace runs unsplit; the workspace query is 0 where no split is planned."""
