@@ -1,9 +1,9 @@
 // Depth-first (pre-order) renumbering of a forest on the device: parent[] -> perm / rank.
 //
 // The reference leaves "DFS ordering so that the nodes of a block share lineage" as an open
-// item (README.md:19-20); the host version is trees.dfs_order.  Integer work, a few launches
-// of N threads each; trees of speculative decoding have a few thousand nodes, so the
-// sibling pass is a tiled all-pairs loop (N^2 / 2 comparisons) rather than a sort.
+// item (README.md:19-20); the host version is trees.dfs_order.  Integer work: one launch of one
+// workgroup for the trees of speculative decoding (a few thousand nodes), six launches of N
+// threads for larger ones; siblings are found through per-parent child lists, not by a sort.
 //
 //   size[i]  nodes in the subtree of i                     (every node adds 1 to each ancestor)
 //   off[i]   sum of size[s] over the siblings s visited before i (roots are siblings of each other)
