@@ -107,6 +107,11 @@ __device__ __forceinline__ uint32_t lds_addr(const void* ptr) {
 // forms the compiler's wait-count pass first drains every outstanding global->LDS
 // transfer (s_waitcnt vmcnt(0)), which would empty the gather ring on every tile.
 // A result is only valid after lds_wait() followed by lds_tie() on it.
+// EVERY result must be tied behind its wait on every path, also one that nobody reads: the data
+// arrives long after the statement, the compiler takes the statement itself as the write, and a
+// result that is dead for the compiler has its registers handed to other values at once, which the
+// late arrival then overwrites (seen on the device: wrong rows in one template instance only,
+// moving with every change of register allocation).
 //
 // ds_read_b64_tr_b16: within each group of 16 lanes, lane i supplies the address of
 // 4 consecutive 16-bit elements (think row i/4, column block i%4 of a 4 x 16 tile)

@@ -14,7 +14,7 @@ from . import _lib
 from .attention import PackedTreeMask, _cache_key, _on_device, _stream_ptr
 
 
-MEDUSA_MAX_CANDIDATES = 16384      # candidate paths fsta_medusa_tree ranks in one launch
+MEDUSA_MAX_CANDIDATES = 1 << 24    # candidate paths the tree builder takes (16384 in one launch, more over a workspace)
 
 
 def _raise_for_status(status: int, max_ancestors: int):
@@ -183,8 +183,11 @@ def medusa_parents_gpu(probs: torch.Tensor, n: int, check: bool = False, status=
     ``n-1`` best paths are kept (ties: shallower first, then smaller ranks) and numbered by
     ``(depth, ranks)``; node 0 is the empty path.  Scores are formed in float64 in the host
     version's multiplication order.  One launch of a HIP kernel on the current stream
-    (``fsta_medusa_tree``; up to 16384 candidate paths = sum of ``topk**d``, e.g. four heads of 10
-    ranks or three of 24; more are refused); with ``dfs_order_gpu``, ``lineage_from_parents_gpu(width=depths + 1)`` and
+    (``fsta_medusa_tree``) for up to 16384 candidate paths = sum of ``topk**d``, e.g. four heads of 10
+    ranks or three of 24; larger sets (up to 2**24 paths, e.g. five or six heads of 10 ranks) go
+    through ``fsta_medusa_tree_ws``: the same selection in about a dozen launches over a workspace
+    of 8 bytes per path taken from torch's allocator.  With ``dfs_order_gpu``,
+    ``lineage_from_parents_gpu(width=depths + 1)`` and
     ``create_fst_attention_kernel_inputs(check=False)`` a tree goes from draft-head probabilities
     to kernel inputs without touching the host.  ``check`` synchronises and raises when a kept
     path's prefix was not kept (probabilities above 1 or not numbers).  ``status``: optional zeroed
@@ -198,8 +201,7 @@ def medusa_parents_gpu(probs: torch.Tensor, n: int, check: bool = False, status=
         raise ValueError(f"n={n} outside [1, {total + 1}] for depths={depths}, topk={topk}")
     if total > MEDUSA_MAX_CANDIDATES or depths * topk > 1024:
         raise ValueError(f"depths={depths}, topk={topk} give {total} candidate paths; the tree builder takes at most "
-                         f"{MEDUSA_MAX_CANDIDATES} (the scores of all candidates live in one workgroup's LDS) and "
-                         f"depths * topk <= 1024")
+                         f"{MEDUSA_MAX_CANDIDATES} and depths * topk <= 1024")
     if probs.dtype not in (torch.float32, torch.float64):
         probs = probs.to(torch.float64)
     probs = probs.contiguous()
@@ -208,9 +210,16 @@ def medusa_parents_gpu(probs: torch.Tensor, n: int, check: bool = False, status=
     parent = torch.empty((n,), dtype=torch.int64, device=dev)
     if status is None:
         status = torch.zeros((1,), dtype=torch.int32, device=dev)
+    code = _lib.F32 if probs.dtype == torch.float32 else _lib.F64
+    need = lib.fsta_medusa_workspace_bytes(depths, topk)
     with _on_device(dev):
-        _lib.check(lib.fsta_medusa_tree(probs.data_ptr(), _lib.F32 if probs.dtype == torch.float32 else _lib.F64,
-                                        depths, topk, n, parent.data_ptr(), status.data_ptr(), _stream_ptr(dev)))
+        if need:
+            work = torch.empty((need,), dtype=torch.uint8, device=dev)     # (stream-ordered: free again after the launches)
+            _lib.check(lib.fsta_medusa_tree_ws(probs.data_ptr(), code, depths, topk, n, parent.data_ptr(), status.data_ptr(),
+                                               work.data_ptr(), need, _stream_ptr(dev)))
+        else:
+            _lib.check(lib.fsta_medusa_tree(probs.data_ptr(), code, depths, topk, n, parent.data_ptr(), status.data_ptr(),
+                                            _stream_ptr(dev)))
     if check and int(status.item()) & _lib.TREE_NOT_PREFIX_CLOSED:
         raise ValueError("the kept paths are not closed under prefixes (probabilities above 1 or not numbers)")
     return parent

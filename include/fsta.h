@@ -323,6 +323,24 @@ int fsta_renumber_parents(const int64_t* parent, const int64_t* rank, int64_t n_
 int fsta_medusa_tree(const void* probs, int32_t probs_dtype, int32_t depths, int32_t topk,
                      int32_t n_nodes, int64_t* parent, uint32_t* status, void* stream);
 
+/*
+ * The same with a device workspace, for more candidate paths than one workgroup's
+ * LDS holds: up to 2^24 paths (e.g. five draft depths of 10 ranks = 111110, six =
+ * 1111110), scores and node ids in the workspace, one launch per step of the
+ * selection (scores, up to eight radix passes, numbering, parents).  Same tree,
+ * bit for bit, as fsta_medusa_tree gives where both apply; no counterpart in the
+ * reference either.
+ *   fsta_medusa_workspace_bytes: bytes of device memory (8-byte aligned) that
+ *     fsta_medusa_tree_ws wants for (depths, topk); 0 when fsta_medusa_tree takes
+ *     the problem (then the workspace may be NULL) or when it is out of range.
+ *   The workspace is free again when the work queued on `stream` has run; calls
+ *   that share one workspace must not overlap.
+ */
+size_t fsta_medusa_workspace_bytes(int32_t depths, int32_t topk);
+int fsta_medusa_tree_ws(const void* probs, int32_t probs_dtype, int32_t depths, int32_t topk,
+                        int32_t n_nodes, int64_t* parent, uint32_t* status,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -150,6 +150,20 @@ def test_tree_builder_rejects_bad_arguments_before_any_gpu_work():
     assert call(8, _lib.F64, 2, 600, 5, 8, 8, None) == _lib.EUNSUPPORTED     # 1200 probabilities
     assert call(8, _lib.F64, 2, 3, 14, 8, 8, None) == _lib.EINVAL            # 12 paths + root < 14 nodes
     assert call(None, _lib.F64, 2, 3, 5, 8, 8, None) == _lib.EINVAL and b"null" in lib.fsta_last_error()
+    # more candidate paths than one workgroup ranks: the workspace variant, with its own checks
+    ws = lambda *a: lib.fsta_medusa_tree_ws(*a)
+    assert lib.fsta_medusa_workspace_bytes(4, 10) == 0                        # 11110 paths: one launch, no workspace
+    need = lib.fsta_medusa_workspace_bytes(5, 10)                             # 111110 paths, 28 workgroups of 4096
+    assert need == 111110 * 8 + 8 * 256 * 4 + 8 * 4 + 28 * 2 * 4
+    assert lib.fsta_medusa_workspace_bytes(8, 10) == 0                        # beyond 2^24 paths: out of range
+    assert ws(8, _lib.F64, 5, 10, 300, 8, 8, None, 0, None) == _lib.EINVAL and b"workspace" in lib.fsta_last_error()
+    assert ws(8, _lib.F64, 5, 10, 300, 8, 8, 64, need - 1, None) == _lib.EINVAL
+    assert ws(8, _lib.F64, 5, 10, 300, 8, 8, 68, need, None) == _lib.EINVAL and b"aligned" in lib.fsta_last_error()
+    assert ws(8, _lib.BF16, 5, 10, 300, 8, 8, 64, need, None) == _lib.EINVAL and b"probs_dtype" in lib.fsta_last_error()
+    assert ws(8, _lib.F64, 8, 10, 300, 8, 8, 64, need, None) == _lib.EUNSUPPORTED
+    assert ws(8, _lib.F64, 2, 200, 50000, 8, 8, 64, 1 << 30, None) == _lib.EINVAL       # 40200 paths + root < 50000 nodes
+    assert ws(None, _lib.F64, 5, 10, 300, 8, 8, 64, need, None) == _lib.EINVAL and b"null" in lib.fsta_last_error()
+    assert ws(8, _lib.F64, 0, 10, 5, 8, 8, None, 0, None) == _lib.EINVAL      # small problems: the checks of fsta_medusa_tree
 
 
 def test_workspace_planning_is_host_arithmetic():

@@ -260,11 +260,61 @@ def test_medusa_tree_built_on_the_gpu_matches_the_host_builder():
     big = trees.medusa_probs(4, 11, 0.3, 12)       # 16104 candidate paths: the largest the kernel takes
     np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(big).cuda(), 1000).cpu().numpy(),
                                   trees.medusa_parents_from_probs(big, 1000))
-    wide = trees.medusa_probs(2, 200, 0.3, 13)     # 40200 paths: more than one launch ranks, refused
-    with pytest.raises(ValueError, match="candidate paths"):
-        medusa_parents_gpu(torch.from_numpy(wide).cuda(), 300)
+    with pytest.raises(ValueError, match="candidate paths"):      # 8 heads of 10 ranks: more than 2**24 paths
+        medusa_parents_gpu(torch.from_numpy(trees.medusa_probs(8, 10, 0.3, 13)).cuda(), 300)
     with pytest.raises(ValueError):                # a deeper path scoring above its prefix
         medusa_parents_gpu(torch.tensor([[0.5, 0.1], [3.0, 0.1]], dtype=torch.float64).cuda(), 2, check=True)
+
+
+
+def _best_paths_host(probs, n):
+    """``trees.medusa_parents_from_probs`` for candidate sets too large to enumerate in Python tuples:
+    the same scores (float64 products from the first rank on), the same order (score descending,
+    then depth, then ranks = candidate index), the same numbering, in numpy."""
+    probs = np.asarray(probs, dtype=np.float64)
+    depths, topk = probs.shape
+    scores, level = [], np.ones(1)
+    for d in range(depths):
+        level = (level[:, None] * probs[d][None, :]).reshape(-1)      # index = ranks read as a base-topk number
+        scores.append(level)
+    flat = np.concatenate(scores)
+    starts = np.concatenate([[0], np.cumsum([len(x) for x in scores])])
+    order = np.lexsort((np.arange(len(flat)), -flat))                 # score descending, ties by index
+    kept = np.sort(order[: n - 1])
+    ids = np.zeros(len(flat), dtype=np.int64)
+    ids[kept] = np.arange(1, n)
+    parent = np.full(n, -1, dtype=np.int64)
+    for c in kept:
+        d = int(np.searchsorted(starts, c, side="right")) - 1
+        parent[ids[c]] = 0 if d == 0 else ids[starts[d - 1] + (c - starts[d]) // topk]
+    return parent
+
+
+def test_medusa_tree_of_more_paths_than_one_workgroup_ranks():
+    """fsta_medusa_tree_ws: scores and ids in a device workspace, a dozen launches; bit-exact against the host."""
+    small = trees.medusa_probs(3, 7, 0.3, 21)       # the numpy restatement against the tuple-based builder
+    np.testing.assert_array_equal(_best_paths_host(small, 120), trees.medusa_parents_from_probs(small, 120))
+    for depths, topk, n, seed in [(5, 10, 1024, 31), (5, 10, 4096, 32), (2, 200, 300, 13), (6, 10, 2048, 33),
+                                  (4, 12, 20000, 34), (3, 40, 64001, 35)]:
+        probs = trees.medusa_probs(depths, topk, 0.3, seed)
+        got = medusa_parents_gpu(torch.from_numpy(probs).cuda(), n).cpu().numpy()
+        np.testing.assert_array_equal(got, _best_paths_host(probs, n), err_msg=f"depths={depths} topk={topk} n={n}")
+    # ties across workgroups: equal probabilities, every path of a depth scores alike
+    uniform = np.full((5, 10), 0.1)
+    for n in (2, 11, 12, 1000, 11111, 50000):
+        got = medusa_parents_gpu(torch.from_numpy(uniform).cuda(), n).cpu().numpy()
+        np.testing.assert_array_equal(got, _best_paths_host(uniform, n), err_msg=f"uniform n={n}")
+    halves = np.tile(np.array([0.5, 0.5, 0.25, 0.25, 0.125, 0.125, 0.0625, 0.0625, 0.03125, 0.03125]), (5, 1))
+    for n in (100, 5000):
+        got = medusa_parents_gpu(torch.from_numpy(halves).cuda(), n).cpu().numpy()
+        np.testing.assert_array_equal(got, _best_paths_host(halves, n), err_msg=f"halves n={n}")
+    p32 = trees.medusa_probs(5, 10, 0.3, 36).astype(np.float32)
+    np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(p32).cuda(), 777).cpu().numpy(),
+                                  _best_paths_host(p32, 777))
+    # the root alone, and every path kept
+    assert medusa_parents_gpu(torch.from_numpy(uniform).cuda(), 1).cpu().tolist() == [-1]
+    full = medusa_parents_gpu(torch.from_numpy(trees.medusa_probs(2, 200, 0.3, 13)).cuda(), 40201).cpu().numpy()
+    np.testing.assert_array_equal(full, _best_paths_host(trees.medusa_probs(2, 200, 0.3, 13), 40201))
 
 
 def test_device_only_pipeline_from_probabilities_to_kernel_inputs():
