@@ -30,6 +30,9 @@ SOURCES = [
     "fsta_attention_prefix.hip",
 ]
 
+# measuring tools that only the instrumented library (--timeline) contains
+TIMELINE_ONLY_SOURCES = ["fsta_probe.hip"]
+
 # packed-fp32 VALU forms are switched off for device code on purpose
 HIPCC_FLAGS = [
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC",
@@ -86,13 +89,15 @@ TIMELINE_LIB_PATH = os.path.join(PKG_DIR, "libfsta_timeline.so")
 def build_library(verbose: bool = True, jobs: int | None = None, timeline: bool = False) -> str:
     """Compiles every source and links ``libfsta.so``; always rebuilds.  ``timeline=True`` builds the
     instrumented variant ``libfsta_timeline.so`` instead (``-DFSTA_TIMELINE``: the matrix-core kernel notes
-    cycle stamps, see ``fstattention_amd/timeline.py``); the regular library is left alone."""
+    cycle stamps, see ``fstattention_amd/timeline.py``, and the issue-rate probe of ``fstattention_amd/mfma_rate.py``
+    is linked in); the regular library is left alone."""
     hipcc = _hipcc()
     obj_dir = OBJ_DIR + ("_timeline" if timeline else "")
     lib_path = TIMELINE_LIB_PATH if timeline else LIB_PATH
     extra = ["-DFSTA_TIMELINE"] if timeline else []
+    sources = SOURCES + (TIMELINE_ONLY_SOURCES if timeline else [])
     os.makedirs(obj_dir, exist_ok=True)
-    jobs = jobs or min(len(SOURCES), os.cpu_count() or 1, 16)
+    jobs = jobs or min(len(sources), os.cpu_count() or 1, 16)
 
     def compile_one(src):
         obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
@@ -100,8 +105,8 @@ def build_library(verbose: bool = True, jobs: int | None = None, timeline: bool 
         return obj, warn
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
-        results = list(pool.map(compile_one, SOURCES))
-    for (obj, warn), src in zip(results, SOURCES):
+        results = list(pool.map(compile_one, sources))
+    for (obj, warn), src in zip(results, sources):
         usage, warn = _split_resource_remarks(warn)
         if src in NO_SCRATCH and not timeline:
             bad = [(name, u) for name, u in usage.items() if u.get("ScratchSize [bytes/lane]", 0)]
