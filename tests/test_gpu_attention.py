@@ -121,6 +121,32 @@ def test_config5_full_size_sampled_rows(order):
     torch.testing.assert_close(o[7:, 63:], one, atol=2e-3, rtol=2e-3)
 
 
+def test_config5_full_size_rows_depend_on_their_ancestors_only():
+    """Size-independent property, all 8 x 64 slices of configuration 5, no oracle: a token attends to itself and
+    to tokens with smaller numbers only (its ancestors), so new K/V values for all rows from r on must leave the
+    outputs and log-sum-exps of the rows below r exactly as they were, and new Q rows from r on likewise."""
+    cfg = trees.config(5)
+    m, d, n = cfg.block_m, cfg.head_dim, cfg.n_nodes
+    lineage, level = trees.lineage_from_parents(cfg.parent)
+    max_anc = trees.required_max_ancestors(cfg.parent, m, 16)
+    inputs = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), m, max_anc)
+    g = torch.Generator(device="cuda").manual_seed(17)
+    q, k, v = (torch.randn((cfg.batch, cfg.heads, n, d), generator=g, device="cuda", dtype=torch.float32)
+               .to(torch.bfloat16) for _ in range(3))
+    scale = 1.0 / math.sqrt(d)
+    call = lambda: fst_attention(q, k, v, *inputs, scale, BLOCK_M=m, MAX_ANCESTORS=max_anc, return_lse=True)
+    o0, lse0 = call()
+    for r in (1, 777, 1280):            # inside a block, and on a block boundary
+        for t in (q, k, v):
+            t[:, :, r:] = torch.randn((cfg.batch, cfg.heads, n - r, d), generator=g, device="cuda",
+                                      dtype=torch.float32).to(torch.bfloat16)
+        o1, lse1 = call()
+        assert torch.equal(o1[:, :, :r], o0[:, :, :r]), f"rows below {r} changed"
+        assert torch.equal(lse1.view(cfg.batch, cfg.heads, n)[:, :, :r], lse0.view(cfg.batch, cfg.heads, n)[:, :, :r])
+        assert not torch.equal(o1[:, :, r:], o0[:, :, r:])
+        o0, lse0 = o1, lse1
+
+
 def test_config5_layer_loop_shares_one_set_of_kernel_inputs():
     """Configuration 5 as it is timed: the kernel inputs are built ONCE on the GPU from the device-resident
     parent array and reused by every layer, each layer with fresh seeded q/k/v (seed = tensor seed + layer).
