@@ -601,7 +601,7 @@ def main():
     long_wall, long_ev = (t["cold_us"] * 1e-6, t["cold_event_us"] * 1e-6) if long_steps == args.steps else \
         time_steps(wl, long_steps, args.warmup, rotate=True, use_graph=use_graph)
     kernel_s = long_ev
-    # Behind a shared prefix the step is up to three launches (tree part, dense prefix kernel, merge) and the dense
+    # Behind a shared prefix the step is two launches (dense prefix kernel, then the tree part which joins) and the dense
     # kernel reads a prefix row once per 128 query rows, not once per block: the per-block byte count of the reference
     # formulation no longer describes what moves, so the roofline figure is taken on q, k, v, o once.
     roofline_bytes = wl.min_traffic_bytes if args.prefix else wl.kv_bytes
@@ -636,7 +636,7 @@ def main():
         "cross_check": {"max_abs_diff_vs_scalar_kernel": max_err, "tol": tol, "ok": ok},
         "roofline": {
             "bound": "hbm",
-            "kernel": kernel_name + (" + prefix_attn_kernel + merge_splits_kernel (whole step)" if args.prefix and wl.key_runs > 1
+            "kernel": kernel_name + (" behind prefix_attn_kernel (whole step: both launches)" if args.prefix and wl.key_runs > 1
                                      else ""),
             "achieved": round(achieved, 2),
             "peak": HBM_PEAK_GBPS,

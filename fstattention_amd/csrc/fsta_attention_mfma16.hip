@@ -741,24 +741,56 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     // per lane; columns go in passes of at most 2*D bytes per row.
     constexpr int kStageStride = D * 2 + 16;     // bytes per staged row (padded against bank conflicts)
     const int first_row = row_base + qgroup * 16;
-    const int hz_out = RUNS ? hz + ksp * p.heads_total : hz;
-    float* const lse_out = RUNS ? p.part_lse : p.lse;
-    void* const o_out = RUNS ? static_cast<void*>(p.part_o) : p.o;
-    const bool out_f32 = RUNS || p.out_f32;
+    // (with key runs: a partial result in the workspace, unless this launch is the one that joins the parts)
+    const bool join = RUNS && p.merge_parts > 0;
+    const bool partial = RUNS && !join;
+    const int hz_out = partial ? hz + ksp * p.heads_total : hz;
+    float* const lse_out = partial ? p.part_lse : p.lse;
+    void* const o_out = partial ? static_cast<void*>(p.part_o) : p.o;
+    const bool out_f32 = partial || p.out_f32;
     auto finish = [&](auto& vals, int col0, unsigned char* stage, bool write_lse) {
         constexpr int kTilesHere = (int)(sizeof(vals) / sizeof(vals[0]));
         const float l_tot = sum_quarters(l_i);
         float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
         if (KV8 && p.v_scale) inv *= p.v_scale[hz];   // O was accumulated on the stored V values
-        if (write_lse) {
-            // the row number is derived again from an opaque copy: kept from the start-up it
-            // would occupy a register pair through the whole kernel
-            int rib = row_in_block;
-            asm volatile("" : "+v"(rib));
-            const int row = row_base + rib;
-            if (row < p.nq && lse_out && g == 0)
-                lse_out[(size_t)hz_out * p.nq + row] = l_tot > 0.f ? m_i + log2f(l_tot) : -INFINITY;
+        float lse_val = l_tot > 0.f ? m_i + log2f(l_tot) : -INFINITY;
+        // the row number is derived again from an opaque copy: kept from the start-up it
+        // would occupy a register pair through the whole kernel
+        int rib = row_in_block;
+        asm volatile("" : "+v"(rib));
+        const int row = row_base + rib;
+        if constexpr (RUNS) {
+            if (join) {
+                // Join with the partial results of the prefix runs (normalised float32 rows with their base-2
+                // log-sum-exps, written by the launch before this one): weights 2^(lse - max), the own part scaled
+                // in place, the others added from memory (this lane's 4 head dims of each of its tiles).
+                const size_t part_rows = (size_t)p.heads_total * p.nq;
+                const size_t mine = (size_t)hz * p.nq + min(row, p.nq - 1);     // (rows past the end: read a real row, store nothing)
+                float mx = lse_val;
+                for (int pp = 1; pp <= p.merge_parts; ++pp) mx = fmaxf(mx, p.part_lse[pp * part_rows + mine]);
+                const float mx_safe = mx == -INFINITY ? 0.f : mx;
+                float wsum = __builtin_amdgcn_exp2f(lse_val - mx_safe);      // exp2(-inf) = 0
+                const float own = wsum * inv;
+#pragma unroll
+                for (int i = 0; i < kTilesHere; ++i)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) vals[i][r] *= own;
+                for (int pp = 1; pp <= p.merge_parts; ++pp) {
+                    const float w = __builtin_amdgcn_exp2f(p.part_lse[pp * part_rows + mine] - mx_safe);
+                    wsum += w;
+                    const float* src = p.part_o + (pp * part_rows + mine) * D + col0 + 4 * g;
+#pragma unroll
+                    for (int i = 0; i < kTilesHere; ++i) {
+                        const f32x4 x = *reinterpret_cast<const f32x4*>(src + 16 * i);
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) vals[i][r] = __builtin_fmaf(w, x[r], vals[i][r]);
+                    }
+                }
+                inv = wsum > 0.f ? 1.f / wsum : 0.f;
+                lse_val = wsum > 0.f ? mx + log2f(wsum) : -INFINITY;
+            }
         }
+        if (write_lse && row < p.nq && lse_out && g == 0) lse_out[(size_t)hz_out * p.nq + row] = lse_val;
         const int rows_valid = p.nq - first_row;
         if (out_f32) {
             constexpr int kPass = kTilesHere < D / 32 ? kTilesHere : D / 32;   // tiles per pass
@@ -882,6 +914,7 @@ int launch_ks(const AttnParams& p, int sub_shift, hipStream_t stream) {
     constexpr size_t kQBytes = (size_t)kWaves * 16 * D * 2;
     const int early = grid <= kCus && !p.part_o && lds + kQBytes <= 160 * 1024 ? 1 : 0;
     if (early) lds += kQBytes;
+    if (p.dry_run) return p.part_o && KS < 0 ? FSTA_EUNSUPPORTED : FSTA_OK;
     if (p.part_o) {
         if constexpr (KS > 0) {
             if (lds > 64 * 1024) {
@@ -933,7 +966,8 @@ template <bool BF16, int D, bool SPLIT>
 int launch_m(const AttnParams& p, hipStream_t stream) {
     // Launches that would leave half of the CUs without a workgroup are cut into half-blocks.
     const int slices_per_xcd = (p.heads_total + kXcds - 1) / kXcds;
-    const bool halve = !p.part_o && kXcds * slices_per_xcd * p.nb * 2 <= kCus;
+    // (also the launch that joins the partial results of a dense prefix: twice the CUs share the reading)
+    const bool halve = (!p.part_o || p.merge_parts > 0) && kXcds * slices_per_xcd * p.nb * 2 <= kCus;
     switch (p.block_m) {
         case 32: return launch_one<BF16, D, 32, SPLIT>(p, 0, stream);
         case 64: return halve ? launch_one<BF16, D, 32, SPLIT>(p, 1, stream) : launch_one<BF16, D, 64, SPLIT>(p, 0, stream);

@@ -47,6 +47,8 @@ namespace {
 constexpr int kKeyTile = 32;        // keys per tile of the attention kernels
 constexpr int kMinRunTiles = 8;     // shortest run of prefix tiles worth a workgroup of its own
 constexpr int kTargetGroups = 512;  // two workgroups per CU
+constexpr int kDenseMinRunTiles = 16;   // the same for the dense prefix kernel, whose partial results the tree part's launch reads back
+                                        // (2048 keys: 4 runs 33.7 us, 8 runs 38.1; 4096 keys: 4 and 8 runs alike)
 
 // How the shared prefix is cut for a launch of the narrow matrix-core kernel: number of runs
 // (1 = no split) and prefix tiles per run.  Depends on the shape and flags only, so that the
@@ -97,7 +99,7 @@ int plan_dense_prefix(int64_t slices, int nq, int nk, int head_dim, int dtype, i
     if (!forced) {
         const int64_t groups = ((slices + 7) / 8) * 8 * ((nq + kDenseRows - 1) / kDenseRows);
         want = (kTargetGroups + groups - 1) / groups;
-        if (want > tiles / kMinRunTiles) want = tiles / kMinRunTiles;
+        if (want > tiles / kDenseMinRunTiles) want = tiles / kDenseMinRunTiles;
         if (want < 1) want = 1;
     }
     if (want > tiles) want = tiles;
@@ -195,11 +197,12 @@ extern "C" int fsta_attention_fwd_ws(const void* q, const void* k, const void* v
     p.key_splits = 1; p.split_tiles = 0; p.part_o = nullptr; p.part_lse = nullptr;
     p.share_tiles = (flags & FSTA_FLAG_SHARE_TILES) ? 1 : 0;
     p.k_scale = nullptr; p.v_scale = nullptr;
+    p.merge_parts = 0; p.dry_run = 0;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (workspace && p.plan) {
-        // a long prefix goes to the dense prefix kernel, run by run; the tree kernel does the tree part only
-        // (slot 0 of the workspace) and one merge joins everything
+        // a long prefix goes to the dense prefix kernel, run by run (slots 1 .. runs of the workspace); the tree
+        // kernel then does the tree part and, in its epilogue, joins it with those partial results into o / lse
         int run_tiles = 0;
         const int runs = plan_dense_prefix(slices, nq, nk, head_dim, dtype, block_m, sm_scale, flags, &run_tiles);
         if (runs > 0 && workspace_bytes >= key_split_bytes(runs + 1, slices, nq, head_dim)) {
@@ -211,13 +214,19 @@ extern "C" int fsta_attention_fwd_ws(const void* q, const void* k, const void* v
             pt.part_lse = pt.part_o + (size_t)(runs + 1) * slices * nq * head_dim;
             pt.key_splits = 1;
             pt.split_tiles = 0;        // no prefix tile for the tree kernel
+            pt.merge_parts = runs;
+            pt.dry_run = 1;            // (would the tree kernel take this shape? asked before anything is launched)
             int rc = launch_attention_mfma16(pt, dtype, head_dim, fast_pv, s);
             if (rc == FSTA_OK) {
-                pt.key_splits = runs;
-                pt.split_tiles = run_tiles;
-                rc = launch_attention_prefix(pt, dtype, head_dim, fast_pv, s);
+                AttnParams pp = pt;
+                pp.dry_run = 0;
+                pp.merge_parts = 0;
+                pp.key_splits = runs;
+                pp.split_tiles = run_tiles;
+                rc = launch_attention_prefix(pp, dtype, head_dim, fast_pv, s);
                 if (rc != FSTA_OK) return rc;
-                return launch_merge_splits(pt.part_o, pt.part_lse, runs + 1, slices * nq, head_dim, o, out_dtype, lse, s);
+                pt.dry_run = 0;
+                return launch_attention_mfma16(pt, dtype, head_dim, fast_pv, s);
             }
             if (rc != FSTA_EUNSUPPORTED) return rc;
             // (ancestor lists too long for the kernel with key runs: the launches below)
@@ -298,5 +307,6 @@ extern "C" int fsta_attention_fwd_kv8(const void* q, const void* k8, const void*
     p.key_splits = 1; p.split_tiles = 0; p.part_o = nullptr; p.part_lse = nullptr;
     p.share_tiles = 0;
     p.k_scale = k_scale; p.v_scale = v_scale;
+    p.merge_parts = 0; p.dry_run = 0;
     return launch_attention_mfma16_kv8(p, dtype, head_dim, static_cast<hipStream_t>(stream));
 }

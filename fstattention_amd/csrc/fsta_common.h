@@ -57,6 +57,11 @@ struct AttnParams {
     int32_t share_tiles;          // tuning: wave pairs of a row group always share the tiles, never the head dimension
     float* part_o;
     float* part_lse;
+    // With merge_parts > 0 the kernel with key runs writes no partial result of its own: it joins its (tree) part
+    // with the partial results in slots 1 .. merge_parts of part_o / part_lse (the dense prefix kernel's, already
+    // written on the stream) and stores the final rows in o / lse.
+    int32_t merge_parts;
+    int32_t dry_run;              // launchers return what they would return without launching anything
     // 8-bit K/V (fsta_attention_fwd_kv8): k and v hold OCP e4m3 bytes; one float32 scale per
     // (batch, head) slice each, or null for 1
     const float* k_scale;

@@ -717,9 +717,9 @@ def test_hip_graph_replays_match_eager_calls():
 
 
 def test_hip_graph_replays_of_key_runs_match_eager_calls():
-    """A long shared prefix cut into runs of keys (tree part, dense prefix kernel and merge: three launches and a
-    workspace from torch's graph-private pool) captured into a HIP graph; replays on new q and new prefix rows
-    must give the eager results."""
+    """A long shared prefix cut into runs of keys (dense prefix kernel, then the tree part that joins: two launches
+    and a workspace from torch's graph-private pool) captured into a HIP graph; replays on new q and new prefix
+    rows must give the eager results."""
     cfg = trees.config(2)
     m, d, prefix = cfg.block_m, cfg.head_dim, 3000
     lineage, level = trees.lineage_from_parents(cfg.parent)
