@@ -187,9 +187,10 @@ int fsta_attention_fwd(const void* q, const void* k, const void* v, void* o, flo
  * ("flash decoding"): when batch * heads * num_blocks workgroups cannot fill
  * the GPU, e.g. one sequence with a long KV cache in front of a small tree, the
  * prefix is read several times faster.  Each run yields a float32 partial
- * result with its log-sum-exp in the workspace; a second kernel joins them into
- * o (and lse).  Results are those of fsta_attention_fwd up to float32 rounding
- * of the join.
+ * result with its log-sum-exp in the workspace; the launch that takes the tree
+ * part (or a small second kernel, where that launch cannot) joins them into o
+ * (and lse).  Results are those of fsta_attention_fwd up to float32 rounding of
+ * the join.
  *   fsta_attention_workspace_bytes: bytes of device memory (256-byte aligned
  *     start) fsta_attention_fwd_ws wants for this problem; 0 when it would not
  *     split (short or no prefix, enough blocks, dtype/shape of the scalar kernel).
