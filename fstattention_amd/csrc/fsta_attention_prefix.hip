@@ -7,8 +7,8 @@
 // groups of 16 query rows and feeds every K / V fragment it reads from LDS to both (half the LDS
 // traffic per product) and no mask words exist.
 // Each workgroup writes a normalised float32 partial result and its base-2 log-sum-exp into the
-// caller's workspace; the tree part (tree kernel, prefix left out) goes into slot 0 and one merge
-// launch joins all parts.  Bound: matrix cores and HBM at once (256 flop per K/V byte at 256 query
+// caller's workspace; the launch of the tree part (tree kernel, prefix left out) reads them back and
+// joins them with its own.  Bound: matrix cores and HBM at once (256 flop per K/V byte at 256 query
 // rows per head against a machine balance of ~310): both have to be kept busy.
 #include <type_traits>
 

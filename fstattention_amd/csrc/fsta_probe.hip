@@ -15,6 +15,21 @@ typedef float probe_f32x4 __attribute__((ext_vector_type(4)));
 typedef float probe_f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
 
+// The shader clock under the load of the loop: s_memtime counts shader cycles, s_memrealtime the constant 100 MHz
+// clock; the first wave of the grid notes how far each got between its first and last instruction, behind the
+// results (out[threads], out[threads + 1]).
+struct ProbeClocks { uint64_t cycles, ticks; };
+__device__ __forceinline__ ProbeClocks probe_clocks() {
+    return ProbeClocks{(uint64_t)__builtin_readcyclecounter(), (uint64_t)__builtin_amdgcn_s_memrealtime()};
+}
+__device__ __forceinline__ void probe_note_clocks(const ProbeClocks& begin, float* out) {
+    const ProbeClocks end = probe_clocks();
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        out[gridDim.x * blockDim.x] = (float)(end.cycles - begin.cycles);
+        out[gridDim.x * blockDim.x + 1] = (float)(end.ticks - begin.ticks);
+    }
+}
+
 // One workgroup of 4 waves per launch slot; every wave runs `iters` rounds of 8 matrix instructions that
 // accumulate into ACCS accumulators in turn (1 = a chain on one accumulator), each followed by VALU
 // independent multiply-adds.  The dynamic LDS size of the launch fixes how many workgroups share a CU.
@@ -22,19 +37,23 @@ template <int SHAPE, int ACCS, int VALU>
 __global__ __launch_bounds__(256) void probe_mfma_kernel(const uint32_t* in, float* out, int iters) {
     extern __shared__ float probe_pad[];
     if (iters < 0) out[0] = probe_pad[threadIdx.x];
+    const ProbeClocks clocks_begin = probe_clocks();
     probe_u32x4 a, b;
     for (int i = 0; i < 4; ++i) { a[i] = in[i * 256 + threadIdx.x]; b[i] = in[(4 + i) * 256 + threadIdx.x]; }
     const probe_bf16x8 A = __builtin_bit_cast(probe_bf16x8, a), B = __builtin_bit_cast(probe_bf16x8, b);
     float s = 0.f;
     float v[8];
     for (int i = 0; i < 8; ++i) v[i] = 1.f + i;
+    // The matrix instructions are written as assembly with the accumulator as an in-out operand: through the
+    // builtin the compiler rotates several accumulators through other registers with dozens of copies per round,
+    // which is then what the loop measures.
     if (SHAPE == 16) {
         probe_f32x4 acc[ACCS];
         for (int i = 0; i < ACCS; ++i) acc[i] = probe_f32x4{0.f, 0.f, 0.f, 0.f};
         for (int it = 0; it < iters; ++it) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                acc[j % ACCS] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A, B, acc[j % ACCS], 0, 0, 0);
+                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc[j % ACCS]) : "v"(A), "v"(B));
 #pragma unroll
                 for (int u = 0; u < VALU; ++u) v[u & 7] = __builtin_fmaf(v[u & 7], 1.0001f, 0.5f);
             }
@@ -47,7 +66,7 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(const uint32_t* in, flo
         for (int it = 0; it < iters; ++it) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                acc[j % ACCS] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A, B, acc[j % ACCS], 0, 0, 0);
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc[j % ACCS]) : "v"(A), "v"(B));
 #pragma unroll
                 for (int u = 0; u < VALU; ++u) v[u & 7] = __builtin_fmaf(v[u & 7], 1.0001f, 0.5f);
             }
@@ -57,6 +76,7 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(const uint32_t* in, flo
     }
     for (int i = 0; i < 8; ++i) s += v[i];
     out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+    probe_note_clocks(clocks_begin, out);
 }
 
 // vector ALU alone: the same multiply-adds without a matrix instruction between them
@@ -64,6 +84,7 @@ template <int VALU>
 __global__ __launch_bounds__(256) void probe_valu_kernel(const uint32_t* in, float* out, int iters) {
     extern __shared__ float probe_pad[];
     if (iters < 0) out[0] = probe_pad[threadIdx.x];
+    const ProbeClocks clocks_begin = probe_clocks();
     float v[8];
     for (int i = 0; i < 8; ++i) v[i] = 1.f + i + (float)in[threadIdx.x];
     for (int it = 0; it < iters; ++it) {
@@ -75,6 +96,7 @@ __global__ __launch_bounds__(256) void probe_valu_kernel(const uint32_t* in, flo
     float s = 0.f;
     for (int i = 0; i < 8; ++i) s += v[i];
     out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+    probe_note_clocks(clocks_begin, out);
 }
 
 template <typename K> int probe_launch(K kernel, const uint32_t* in, float* out, int iters, int waves_per_simd, hipStream_t s) {
@@ -92,7 +114,7 @@ template <typename K> int probe_launch(K kernel, const uint32_t* in, float* out,
 using namespace fsta;
 
 // shape 16 (16x16x32) or 32 (32x32x16), 0 = vector ALU only; accumulators 1, 2, 4 or 8; 0, 2, 4 or 8 multiply-adds
-// per matrix instruction; 1 or 2 waves per SIMD.  `in`: 2048 uint32 (bf16 pairs), `out`: 2 * 256 * 256 floats.
+// per matrix instruction; 1 or 2 waves per SIMD.  `in`: 2048 uint32 (bf16 pairs), `out`: 2 * 256 * 256 + 2 floats.
 extern "C" int fsta_probe_mfma_rate(int32_t shape, int32_t accumulators, int32_t valu, int32_t waves_per_simd,
                                     int32_t iters, const uint32_t* in, float* out, void* stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
