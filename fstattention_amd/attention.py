@@ -6,6 +6,7 @@ current torch stream; torch only owns the memory.
 """
 from __future__ import annotations
 
+import weakref
 from typing import NamedTuple, Optional
 
 import torch
@@ -115,7 +116,7 @@ def _version(t: torch.Tensor):
 
 
 def _cache_key(ancestor_idx, ancestor_mask, leaf_idx):
-    """What a packed copy kept on ``ancestor_mask`` was made from, or None when in-place edits of
+    """What a packed copy remembered for ``ancestor_mask`` was made from, or None when in-place edits of
     one of the three tensors could not be noticed."""
     versions = (_version(ancestor_mask), _version(ancestor_idx), _version(leaf_idx))
     if None in versions:
@@ -123,28 +124,47 @@ def _cache_key(ancestor_idx, ancestor_mask, leaf_idx):
     return versions + (ancestor_idx.data_ptr(), leaf_idx.data_ptr(), tuple(ancestor_mask.shape))
 
 
+# Packed copies of bool masks, by the identity of the mask tensor: id -> (weak reference, key, packed).  The
+# entry goes when the tensor does (weakref.finalize), so nothing is kept alive and nothing is hung on the
+# caller's objects.
+_PACKED: dict = {}
+
+
+def remember_packed(ancestor_mask: torch.Tensor, key, packed: PackedTreeMask) -> None:
+    """Notes `packed` as the packed form of the bool tensor `ancestor_mask` in the state `key` describes."""
+    ident = id(ancestor_mask)
+    if ident not in _PACKED or _PACKED[ident][0]() is not ancestor_mask:
+        weakref.finalize(ancestor_mask, _PACKED.pop, ident, None)
+    _PACKED[ident] = (weakref.ref(ancestor_mask), key, packed)
+
+
+def recall_packed(ancestor_mask: torch.Tensor):
+    """(key, packed) noted for this very tensor object, or None."""
+    entry = _PACKED.get(id(ancestor_mask))
+    if entry is None or entry[0]() is not ancestor_mask:
+        return None
+    return entry[1], entry[2]
+
+
 def _packed_for(ancestor_idx: torch.Tensor, ancestor_mask, leaf_idx: torch.Tensor, nk: int) -> PackedTreeMask:
-    """Packed mask and block plan of a bool tensor, remembered on the tensor object.
+    """Packed mask and block plan of a bool tensor, remembered per tensor object.
 
     The kernel inputs are built once per decoding step and reused by every
-    layer; the packed copy is kept as an attribute of ``ancestor_mask`` and
-    dropped when one of the three tensors has been written to since (torch's version
-    counters), ``ancestor_idx`` or ``leaf_idx`` is a different tensor, or K/V have another number
-    of rows than the plan was made for.  Tensors without version counters (inference mode) are
-    packed on every call; pass a :class:`PackedTreeMask` to avoid that.
+    layer; the packed copy is kept in a module-level table under the identity of ``ancestor_mask``
+    (dropped with the tensor) and replaced when one of the three tensors has been written to since
+    (torch's version counters), ``ancestor_idx`` or ``leaf_idx`` is a different tensor, or K/V have
+    another number of rows than the plan was made for.  Tensors without version counters (inference
+    mode) are packed on every call; pass a :class:`PackedTreeMask` to avoid that.
     """
     if isinstance(ancestor_mask, PackedTreeMask):
         return ancestor_mask
     key = _cache_key(ancestor_idx, ancestor_mask, leaf_idx)
-    cached = getattr(ancestor_mask, "_fsta_packed", None) if key is not None else None
+    cached = recall_packed(ancestor_mask) if key is not None else None
     if cached is not None and cached[0] == key and cached[1].key_limit in (None, nk):
         return cached[1]
     packed = pack_tree_mask(ancestor_idx, ancestor_mask, leaf_idx, nk)
     if key is not None:
-        try:
-            ancestor_mask._fsta_packed = (key, packed)
-        except AttributeError:
-            pass
+        remember_packed(ancestor_mask, key, packed)
     return packed
 
 

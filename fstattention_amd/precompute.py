@@ -11,7 +11,7 @@ from typing import Optional
 import torch
 
 from . import _lib
-from .attention import PackedTreeMask, _cache_key, _on_device, _stream_ptr
+from .attention import PackedTreeMask, _cache_key, _on_device, _stream_ptr, remember_packed
 
 
 MEDUSA_MAX_CANDIDATES = 1 << 24    # candidate paths the tree builder takes (16384 in one launch, more over a workspace)
@@ -92,7 +92,7 @@ def create_fst_attention_kernel_inputs(lineage, level_lookup, block_m=64, max_an
     else:
         key = _cache_key(a_idx, a_mask, l_idx) if want_bool_mask else None
         if key is not None:     # (tensors made in inference mode keep no edit counters: packed per call instead)
-            a_mask._fsta_packed = (key, packed)
+            remember_packed(a_mask, key, packed)
         out = (a_idx, a_mask if want_bool_mask else packed, l_idx)
     return out if check else out + (status,)
 

@@ -13,6 +13,7 @@ import torch
 from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, fst_attention,
                               lineage_from_parents_gpu, merge_attention_states, renumber_parents_gpu, shift_for_prefix,
                               trees)
+from fstattention_amd.attention import recall_packed
 from helpers import TOL, assert_close, dense_oracle, oracle_inputs, rand_qkv
 from oracle import tree_precompute as tp
 
@@ -491,9 +492,11 @@ def test_packed_inputs_follow_a_prefix_shift_and_inference_mode():
             o = fst_attention(qd, kd, vd, a_sh, packed_sh, l_sh, scale, BLOCK_M=m, MAX_ANCESTORS=max_anc,
                               out_dtype=torch.float32)
             assert_close(o, want, torch.bfloat16, f"packed inputs behind a prefix, inference={inference}")
-            # bool mask: packed by fst_attention itself (kept on the tensor outside inference mode)
+            # bool mask: packed by fst_attention itself (remembered for the tensor outside inference mode, and
+            # never as an attribute of the caller's tensor)
             a_idx, a_mask, l_idx = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), m, max_anc)
-            assert hasattr(a_mask, "_fsta_packed") != inference
+            assert (recall_packed(a_mask) is not None) != inference
+            assert not hasattr(a_mask, "_fsta_packed")
             a_sh, l_sh = shift_for_prefix(a_idx, l_idx, prefix)
             for _ in range(2):
                 o = fst_attention(qd, kd, vd, a_sh, a_mask, l_sh, scale, BLOCK_M=m, MAX_ANCESTORS=max_anc,

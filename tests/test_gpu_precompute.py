@@ -6,6 +6,7 @@ import torch
 from conftest import golden_cases
 from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, lineage_from_parents_gpu,
                               medusa_parents_gpu, pack_tree_mask, renumber_parents_gpu, trees)
+from fstattention_amd.attention import recall_packed
 from oracle import tree_precompute as tp
 
 pytestmark = pytest.mark.gpu
@@ -119,7 +120,7 @@ def test_packed_mask_matches_bool_mask():
     lineage, level = trees.lineage_from_parents(parent)
     max_anc = trees.required_max_ancestors(parent, 64, 1)
     a_idx, a_mask, l_idx = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), 64, max_anc)
-    from_precompute = a_mask._fsta_packed[1]
+    from_precompute = recall_packed(a_mask)[1]
     repacked = pack_tree_mask(a_idx, a_mask)
     assert torch.equal(from_precompute.mask_bits, repacked.mask_bits)
     assert torch.equal(from_precompute.anc_count, repacked.anc_count)
@@ -140,7 +141,7 @@ def test_block_plan_matches_the_lists(block_m, n, window):
     lineage, level = trees.lineage_from_parents(parent)
     max_anc = trees.required_max_ancestors(parent, block_m, 16)
     a_idx, a_mask, l_idx = create_fst_attention_kernel_inputs(lineage.cuda(), level.cuda(), block_m, max_anc)
-    made = a_mask._fsta_packed[1]
+    made = recall_packed(a_mask)[1]
     nb = a_idx.shape[0]
     want, care = expected_plan(a_idx.cpu().numpy(), a_mask.cpu().numpy(), l_idx.cpu().numpy())
     for label, packed in (("precompute", made), ("pack", pack_tree_mask(a_idx, a_mask, l_idx))):
