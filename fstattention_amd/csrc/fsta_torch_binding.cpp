@@ -1,5 +1,6 @@
-// PyTorch operator registration of the attention entry point (host code only, no kernels):
+// PyTorch operator registration of the two entry points of the path (host code only, no kernels):
 //   torch.ops.fsta.attention_fwd(...)  ->  fsta_attention_fwd_ws / fsta_attention_fwd_kv8 of libfsta.so
+//   torch.ops.fsta.precompute(...)     ->  fsta_precompute (reference utils.py:104-129)
 // on torch's current HIP stream of the tensors' device.  It does in C++ what the operator wrapper of
 // reference fstattention.py:153-181 does in Python (shape checks, allocation of o and L, launch), so
 // that an eager caller pays the dispatcher and one allocation per call instead of a page of Python.
@@ -113,14 +114,68 @@ std::tuple<at::Tensor, at::Tensor> attention_fwd(const at::Tensor& q, const at::
     return {o, lse};
 }
 
+// lineage [N, W] int64 (contiguous; written to when mutate_lineage, as utils.py:124-125 writes to the caller's
+// tensor), level_lookup [N] int64, on the GPU.  Returns the three tensors of the reference (ancestor_mask empty
+// unless want_bool_mask), the packed mask, the per-block ancestor counts, the block plan (empty for block sizes
+// the matrix-core kernels do not take) and the status word (FSTA_PRE_* bits; the caller's own zeroed word if one
+// was passed, so that the stages of a front-end chain share one).
+std::tuple<at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor, at::Tensor> precompute(
+    at::Tensor& lineage, const at::Tensor& level_lookup, int64_t block_m, int64_t max_ancestors, bool mutate_lineage,
+    bool want_bool_mask, const c10::optional<at::Tensor>& status) {
+    TORCH_CHECK_VALUE(lineage.dim() == 2 && level_lookup.dim() == 1 && level_lookup.size(0) == lineage.size(0),
+                      "lineage must be [N, W] and level_lookup [N]");
+    TORCH_CHECK_VALUE(lineage.scalar_type() == at::kLong && level_lookup.scalar_type() == at::kLong,
+                      "lineage and level_lookup must be int64");
+    TORCH_CHECK_VALUE(lineage.is_cuda() && level_lookup.device() == lineage.device(),
+                      "the precompute runs on the GPU only (no CPU fallback); both tensors on one device");
+    TORCH_CHECK_VALUE(lineage.is_contiguous() && level_lookup.is_contiguous(), "lineage and level_lookup must be contiguous");
+    TORCH_CHECK_VALUE(block_m > 0 && max_ancestors > 0, "block_m and max_ancestors must be positive");
+    const int64_t n = lineage.size(0), width = lineage.size(1);
+    const int64_t nb = (n + block_m - 1) / block_m;
+    const auto i64 = lineage.options();
+    const auto i32 = lineage.options().dtype(at::kInt);
+    at::Tensor a_idx = at::empty({nb, max_ancestors}, i64);
+    at::Tensor a_mask = want_bool_mask ? at::empty({nb, block_m, max_ancestors}, lineage.options().dtype(at::kBool)) : at::Tensor();
+    at::Tensor l_idx = at::empty({nb, block_m}, i64);
+    at::Tensor bits = at::empty({nb, (int64_t)fsta_mask_words((int32_t)max_ancestors), block_m}, i32);
+    at::Tensor count = at::empty({nb}, i32);
+    const size_t plan_bytes = fsta_block_plan_bytes((int32_t)nb, (int32_t)block_m, (int32_t)max_ancestors);
+    at::Tensor plan = plan_bytes ? at::empty({(int64_t)(plan_bytes / 4)}, i32) : at::Tensor();
+    at::Tensor st;
+    if (status.has_value() && status->defined()) {
+        TORCH_CHECK_VALUE(status->scalar_type() == at::kInt && status->numel() == 1 && status->device() == lineage.device(),
+                          "status must be one int32 on the tensors' device");
+        st = *status;
+    } else {
+        st = at::zeros({1}, i32);
+    }
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(lineage.device());
+    const hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(lineage.device().index()).stream();
+    check_rc(fsta_precompute(lineage.data_ptr<int64_t>(), level_lookup.data_ptr<int64_t>(), n, width, (int32_t)block_m,
+                             (int32_t)max_ancestors, mutate_lineage ? 1 : 0, a_idx.data_ptr<int64_t>(),
+                             want_bool_mask ? static_cast<uint8_t*>(a_mask.data_ptr()) : nullptr, l_idx.data_ptr<int64_t>(),
+                             static_cast<uint32_t*>(bits.data_ptr()), count.data_ptr<int32_t>(),
+                             plan_bytes ? static_cast<uint32_t*>(plan.data_ptr()) : nullptr,
+                             static_cast<uint32_t*>(st.data_ptr()), stream));
+    return {a_idx, a_mask, l_idx, bits, count, plan, st};
+}
+
 }  // namespace
 
 TORCH_LIBRARY(fsta, m) {
+    m.def("precompute(Tensor(a!) lineage, Tensor level_lookup, int block_m, int max_ancestors, bool mutate_lineage, "
+          "bool want_bool_mask, Tensor(b!)? status) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)");
     m.def("attention_fwd(Tensor q, Tensor k, Tensor v, Tensor ancestor_idx, Tensor mask_bits, Tensor anc_count, "
           "Tensor leaf_idx, Tensor? plan, int key_shift, float sm_scale, int block_m, int max_ancestors, "
           "int out_dtype_code, bool return_lse, int flags, Tensor? k_scale, Tensor? v_scale) -> (Tensor, Tensor)");
 }
 
-TORCH_LIBRARY_IMPL(fsta, CUDA, m) { m.impl("attention_fwd", &attention_fwd); }
+TORCH_LIBRARY_IMPL(fsta, CUDA, m) {
+    m.impl("attention_fwd", &attention_fwd);
+    m.impl("precompute", &precompute);
+}
 // tensors that all live on the host end up here: same message as for a mixed call
-TORCH_LIBRARY_IMPL(fsta, CPU, m) { m.impl("attention_fwd", &attention_fwd); }
+TORCH_LIBRARY_IMPL(fsta, CPU, m) {
+    m.impl("attention_fwd", &attention_fwd);
+    m.impl("precompute", &precompute);
+}

@@ -53,7 +53,6 @@ def create_fst_attention_kernel_inputs(lineage, level_lookup, block_m=64, max_an
         raise ValueError("lineage and level_lookup must be int64")
     block_m = int(block_m)
     max_ancestors = int(max_ancestors)
-    lib = _lib.load()
     on_host = not lineage.is_cuda
     if on_host:
         if not torch.cuda.is_available():
@@ -64,24 +63,13 @@ def create_fst_attention_kernel_inputs(lineage, level_lookup, block_m=64, max_an
         dev = lineage.device
     lin = lineage.to(dev).contiguous()
     lvl = level_lookup.to(dev).contiguous()
-    n, width = lin.shape
-    nb = -(-n // block_m)
-    words = (max_ancestors + 31) // 32
-    a_idx = torch.empty((nb, max_ancestors), dtype=torch.int64, device=dev)
-    a_mask = torch.empty((nb, block_m, max_ancestors), dtype=torch.bool, device=dev) if want_bool_mask else None
-    l_idx = torch.empty((nb, block_m), dtype=torch.int64, device=dev)
-    bits = torch.empty((nb, words, block_m), dtype=torch.int32, device=dev)
-    count = torch.empty((nb,), dtype=torch.int32, device=dev)
-    plan_bytes = lib.fsta_block_plan_bytes(nb, block_m, max_ancestors)
-    plan = torch.empty((plan_bytes // 4,), dtype=torch.int32, device=dev) if plan_bytes else None
-    if status is None:
-        status = torch.zeros((1,), dtype=torch.int32, device=dev)
-    with _on_device(dev):
-        _lib.check(lib.fsta_precompute(
-            lin.data_ptr(), lvl.data_ptr(), n, width, block_m, max_ancestors, int(mutate_lineage),
-            a_idx.data_ptr(), a_mask.data_ptr() if want_bool_mask else None, l_idx.data_ptr(),
-            bits.data_ptr(), count.data_ptr(), plan.data_ptr() if plan is not None else None,
-            status.data_ptr(), _stream_ptr(dev)))
+    # one operator call (csrc/fsta_torch_binding.cpp): allocations, stream, device guard and the launch in C++
+    a_idx, a_mask, l_idx, bits, count, plan, status = _lib.load_torch_ops().precompute(
+        lin, lvl, block_m, max_ancestors, bool(mutate_lineage), bool(want_bool_mask), status)
+    if not want_bool_mask:
+        a_mask = None
+    if plan is not None and plan.numel() == 0:      # (block sizes the matrix-core kernels do not take have no plan)
+        plan = None
     if check:
         _raise_for_status(int(status.item()), max_ancestors)
     if mutate_lineage and lin.data_ptr() != lineage.data_ptr():
