@@ -227,3 +227,25 @@ def test_python_entry_points_refuse_to_run_without_a_gpu_path():
         lineage, level = trees.lineage_from_parents([-1, 0, 1])
         with pytest.raises(RuntimeError, match="GPU"):
             create_fst_attention_kernel_inputs(lineage, level, 4, 4)
+
+
+def test_operator_library_registers_both_operators_and_rejects_host_tensors():
+    """``_fsta_torch.so`` registers ``fsta::attention_fwd`` and ``fsta::precompute`` with torch's dispatcher;
+    both check their arguments on the host and refuse tensors that are not on the GPU."""
+    import torch
+    if not os.path.exists(_lib.TORCH_OPS_PATH):
+        pytest.fail(f"{_lib.TORCH_OPS_PATH} has not been built (python -m fstattention_amd.build)")
+    ops = _lib.load_torch_ops()
+    pre = ops.precompute.default._schema
+    assert [a.name for a in pre.arguments] == ["lineage", "level_lookup", "block_m", "max_ancestors", "mutate_lineage",
+                                               "want_bool_mask", "status"]
+    assert len(pre.returns) == 7
+    assert pre.arguments[0].alias_info is not None and pre.arguments[0].alias_info.is_write   # lineage is written
+    fwd = ops.attention_fwd.default._schema
+    assert [a.name for a in fwd.arguments][:6] == ["q", "k", "v", "ancestor_idx", "mask_bits", "anc_count"]
+    lineage = torch.tensor([[0, -1], [0, 1]], dtype=torch.int64)
+    level = torch.tensor([0, 1], dtype=torch.int64)
+    with pytest.raises(ValueError, match="GPU"):
+        ops.precompute(lineage, level, 2, 2, True, True, None)
+    with pytest.raises(ValueError, match="int64"):
+        ops.precompute(lineage.int(), level, 2, 2, True, True, None)
