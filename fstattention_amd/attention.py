@@ -226,6 +226,16 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
         if (ancestor_mask.block_m, ancestor_mask.max_ancestors) != (BLOCK_M, MAX_ANCESTORS):
             raise ValueError("packed mask was built for another block size / ancestor count")
         packed = ancestor_mask
+        # A plan made by the tree precompute names tree nodes; with K/V laid out as [prefix | tree] the
+        # only shift that makes it agree with index tensors shifted by ``shift_for_prefix`` is the
+        # prefix length.  Shifted tensors passed with the unshifted packed inputs (the third return
+        # value of ``shift_for_prefix`` dropped) would otherwise gather prefix rows as ancestors in
+        # the kernels that read the plan and the right rows in those that read the lists.
+        if packed.plan is not None and packed.key_limit is None and q.dim() == 4 and k.dim() == 4 and \
+                packed.key_shift != k.shape[2] - q.shape[2]:
+            raise ValueError(f"packed kernel inputs carry key_shift={packed.key_shift} but k has "
+                             f"{k.shape[2] - q.shape[2]} prefix rows in front of the tree: pass the third value "
+                             "returned by shift_for_prefix(ancestor_idx, leaf_idx, prefix, packed)")
     else:
         if ancestor_mask.dim() != 3 or ancestor_mask.shape[1] != BLOCK_M or ancestor_mask.shape[2] != MAX_ANCESTORS or \
                 ancestor_mask.shape[0] != ancestor_idx.shape[0]:

@@ -28,10 +28,8 @@ SOURCES = [
     "fsta_attention_mfma.hip",
     "fsta_attention_mfma16.hip",
     "fsta_attention_prefix.hip",
+    "fsta_roofline.hip",
 ]
-
-# measuring tools that only the instrumented library (--timeline) contains
-TIMELINE_ONLY_SOURCES = ["fsta_probe.hip"]
 
 # packed-fp32 VALU forms are switched off for device code on purpose
 HIPCC_FLAGS = [
@@ -89,13 +87,12 @@ TIMELINE_LIB_PATH = os.path.join(PKG_DIR, "libfsta_timeline.so")
 def build_library(verbose: bool = True, jobs: int | None = None, timeline: bool = False) -> str:
     """Compiles every source and links ``libfsta.so``; always rebuilds.  ``timeline=True`` builds the
     instrumented variant ``libfsta_timeline.so`` instead (``-DFSTA_TIMELINE``: the matrix-core kernel notes
-    cycle stamps, see ``fstattention_amd/timeline.py``, and the issue-rate probe of ``fstattention_amd/mfma_rate.py``
-    is linked in); the regular library is left alone."""
+    cycle stamps, see ``fstattention_amd/timeline.py``); the regular library is left alone."""
     hipcc = _hipcc()
     obj_dir = OBJ_DIR + ("_timeline" if timeline else "")
     lib_path = TIMELINE_LIB_PATH if timeline else LIB_PATH
     extra = ["-DFSTA_TIMELINE"] if timeline else []
-    sources = SOURCES + (TIMELINE_ONLY_SOURCES if timeline else [])
+    sources = SOURCES
     os.makedirs(obj_dir, exist_ok=True)
     jobs = jobs or min(len(sources), os.cpu_count() or 1, 16)
 

@@ -61,14 +61,16 @@ __device__ __forceinline__ int32_t checked_parent(const int64_t* __restrict__ pa
     return (p >= -1 && p < i) ? (int32_t)p : -2;   // -2: malformed entry
 }
 
-__global__ __launch_bounds__(kOrderThreads) void order_init_kernel(int32_t n, int32_t* size, int32_t* kids) {
+__global__ __launch_bounds__(kOrderThreads) void order_init_kernel(int32_t n, int32_t* size, int32_t* kids, int32_t* bad) {
     const int32_t i = blockIdx.x * kOrderThreads + threadIdx.x;
     if (i < n) size[i] = 1;
     if (i <= n) kids[i] = 0;
+    if (i == 0) *bad = 0;
 }
 
 __global__ __launch_bounds__(kOrderThreads) void order_sizes_kernel(const int64_t* __restrict__ parent, int32_t n,
-                                                                    int32_t* size, int32_t* kids, uint32_t* status) {
+                                                                    int32_t* size, int32_t* kids, int32_t* bad,
+                                                                    uint32_t* status) {
     const int32_t i = blockIdx.x * kOrderThreads + threadIdx.x;
     if (i >= n) return;
     int32_t a = checked_parent(parent, i);
@@ -85,7 +87,12 @@ __global__ __launch_bounds__(kOrderThreads) void order_sizes_kernel(const int64_
         }
         a = checked_parent(parent, a);
     }
-    if (a < -1) atomicOr(status, FSTA_PRE_BAD_NODE_ID);
+    // `bad` is this call's own flag (the status word may already carry bits of an earlier stage of a
+    // front-end chain, which say nothing about this parent array)
+    if (a < -1) {
+        atomicOr(status, FSTA_PRE_BAD_NODE_ID);
+        atomicOr(bad, 1);
+    }
 }
 
 constexpr int kScanThreads = 1024;
@@ -154,10 +161,10 @@ __global__ __launch_bounds__(kOrderThreads) void order_offsets_kernel(const int6
 __global__ __launch_bounds__(kOrderThreads) void order_finish_kernel(const int64_t* __restrict__ parent, int32_t n,
                                                                      const int32_t* __restrict__ off, int64_t* __restrict__ perm,
                                                                      int64_t* __restrict__ rank,
-                                                                     const uint32_t* status) {
+                                                                     const int32_t* bad) {
     const int32_t i = blockIdx.x * kOrderThreads + threadIdx.x;
     if (i >= n) return;
-    if (*status) {      // malformed parent array: identity, the caller reads the status word
+    if (*bad) {      // malformed parent array: identity, the caller reads the status word
         perm[i] = i;
         rank[i] = i;
         return;
@@ -318,15 +325,16 @@ int dfs_order_launch(const int64_t* parent, int64_t n_nodes, int32_t light_first
     int32_t* first = kids + n + 1;             // [n + 1]
     int32_t* cursor = first + n + 1;           // [n + 1]
     int32_t* child = cursor + n + 1;           // [n]
+    int32_t* bad = child + n;                  // [1] this call found a malformed parent entry
     const unsigned blocks = (unsigned)((n_nodes + kOrderThreads) / kOrderThreads);   // covers n + 1 entries
     // (every array is written by a kernel before it is read: nothing of an earlier call survives)
-    hipLaunchKernelGGL(order_init_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, n, size, kids);
-    hipLaunchKernelGGL(order_sizes_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, parent, n, size, kids, status);
+    hipLaunchKernelGGL(order_init_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, n, size, kids, bad);
+    hipLaunchKernelGGL(order_sizes_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, parent, n, size, kids, bad, status);
     hipLaunchKernelGGL(order_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, n, kids, first, cursor);
     hipLaunchKernelGGL(order_fill_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, parent, n, cursor, child);
     hipLaunchKernelGGL(order_offsets_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, parent, n, light_first ? 1 : 0,
                        size, kids, first, child, off);
-    hipLaunchKernelGGL(order_finish_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, parent, n, off, perm, rank, status);
+    hipLaunchKernelGGL(order_finish_kernel, dim3(blocks), dim3(kOrderThreads), 0, s, parent, n, off, perm, rank, bad);
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
 }

@@ -199,6 +199,10 @@ int fsta_attention_fwd(const void* q, const void* k, const void* v, void* o, flo
  *     fsta_attention_fwd).  The workspace is free again when the work queued on
  *     `stream` has run; calls that share one workspace must not overlap.
  * `flags` must be the same in both calls; FSTA_FLAG_KEY_SPLITS(n) forces n runs.
+ * Both the runs of keys and the dense prefix kernel read the block plan: a call
+ * with block_plan = NULL ignores the workspace and walks the prefix unsplit in one
+ * launch (correct, slower), whatever fsta_attention_workspace_bytes said -- that
+ * function has no plan argument and answers for a caller that passes one.
  */
 size_t fsta_attention_workspace_bytes(int32_t batch, int32_t heads, int32_t nq, int32_t nk,
                                       int32_t head_dim, int32_t dtype, int32_t block_m,
@@ -254,9 +258,10 @@ int fsta_lineage_from_parents(const int64_t* parent, int64_t n_nodes, int64_t wi
  * perm[new_id] = old_id and rank[old_id] = new_id, both int64 [n_nodes].
  * Siblings (and roots) are visited by ascending id, or smallest subtree first
  * (ties by id) when light_first != 0.  workspace:
- * FSTA_DFS_ORDER_WORKSPACE_INTS(n_nodes) int32 of device scratch.  `status` (zero
- * on entry) gets FSTA_PRE_BAD_NODE_ID for a parent entry outside [-1, i); perm
- * and rank are then the identity.  n_nodes <= FSTA_DFS_ORDER_MAX_NODES (2^17, the
+ * FSTA_DFS_ORDER_WORKSPACE_INTS(n_nodes) int32 of device scratch.  `status` gets
+ * FSTA_PRE_BAD_NODE_ID for a parent entry outside [-1, i); perm and rank are then
+ * the identity.  Bits already set in `status` on entry (earlier stages of a
+ * front-end chain may share the word) are left alone and do not change the result.  n_nodes <= FSTA_DFS_ORDER_MAX_NODES (2^17, the
  * largest entry of the reference's size table, utils.py:4-13).  Work is
  * O(n_nodes * depth + sum over parents of children^2).
  */
@@ -275,7 +280,10 @@ int fsta_dfs_order(const int64_t* parent, int64_t n_nodes, int32_t light_first, 
  * larger trees are refused with FSTA_EUNSUPPORTED.  All calls on one GPU share
  * that GPU's array: calls that overlap on one GPU (two streams, two threads)
  * race, queue them on one stream or order them with events.  The first call on
- * a device looks the array's address up (no memory is allocated).
+ * a device looks the array's address up (hipGetSymbolAddress under a mutex; no
+ * memory is allocated): make that first call outside stream capture, later calls
+ * may be captured.  The array used is the one of the CURRENT device, which must be
+ * the device `stream` belongs to.
  */
 #define FSTA_DFS_ORDER_STATIC_MAX_NODES 16384
 int fsta_dfs_order_static(const int64_t* parent, int64_t n_nodes, int32_t light_first, int64_t* perm,
@@ -341,6 +349,19 @@ size_t fsta_medusa_workspace_bytes(int32_t depths, int32_t topk);
 int fsta_medusa_tree_ws(const void* probs, int32_t probs_dtype, int32_t depths, int32_t topk,
                         int32_t n_nodes, int64_t* parent, uint32_t* status,
                         void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Measuring aids (no counterpart in the reference; bench.py reports them beside
+ * the attention kernels' figures as this GPU's own ceilings).
+ *   fsta_probe_empty_launch: one launch of a kernel that does nothing, `workgroups`
+ *     workgroups of `threads` threads: what a launch of that shape costs by itself.
+ *   fsta_probe_hbm_read: a kernel that only reads: `bytes` (a multiple of 16) from
+ *     src (16-byte aligned), 16 bytes per lane, consecutive lanes consecutive
+ *     addresses, eight loads per lane in flight, `workgroups` workgroups of 256
+ *     threads; `sink` (may be NULL) is never written in practice.
+ */
+int fsta_probe_empty_launch(int32_t workgroups, int32_t threads, void* stream);
+int fsta_probe_hbm_read(const void* src, size_t bytes, int32_t workgroups, uint32_t* sink, void* stream);
 
 #ifdef __cplusplus
 }

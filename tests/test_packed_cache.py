@@ -44,3 +44,21 @@ def test_prefix_shift_travels_with_the_packed_inputs():
     assert len(shift_for_prefix(idx, leaf, 100)) == 2
     from_tree = PackedTreeMask(torch.zeros(1), torch.zeros(1), 32, 8, torch.zeros(1))
     assert shift_for_prefix(idx, leaf, 7, from_tree)[2].key_limit is None
+
+
+def test_shifted_lists_with_unshifted_packed_inputs_are_refused():
+    """Index tensors moved behind a prefix must come with the packed inputs ``shift_for_prefix`` returns:
+    a plan of the tree precompute whose shift is not the prefix length is refused before anything runs."""
+    import pytest
+    from fstattention_amd import fst_attention
+    idx, _, leaf = _lists()
+    from_tree = PackedTreeMask(torch.zeros(1), torch.zeros(1), 32, 8, torch.zeros(1))      # key_shift 0, tree plan
+    q = torch.zeros((1, 1, 64, 64))
+    kv = torch.zeros((1, 1, 64 + 100, 64))
+    a_sh, l_sh = shift_for_prefix(idx, leaf, 100)
+    with pytest.raises(ValueError, match="key_shift"):
+        fst_attention(q, kv, kv, a_sh, from_tree, l_sh, 1.0, BLOCK_M=32, MAX_ANCESTORS=8)
+    # the other way round: a shifted plan in front of K/V without the prefix
+    _, _, shifted = shift_for_prefix(idx, leaf, 100, from_tree)
+    with pytest.raises(ValueError, match="key_shift"):
+        fst_attention(q, q, q, idx, shifted, leaf, 1.0, BLOCK_M=32, MAX_ANCESTORS=8)
