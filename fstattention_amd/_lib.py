@@ -9,7 +9,7 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libfsta.so"
 
 F32, F16, BF16, F64 = 0, 1, 2, 3
 OK, EINVAL, EUNSUPPORTED, EHIP = 0, -1, -2, -3
-FLAG_FAST_PV, FLAG_GENERIC, FLAG_WIDE_WAVES, FLAG_SHARE_TILES = 1, 2, 4, 8
+FLAG_FAST_PV, FLAG_GENERIC, FLAG_WIDE_WAVES, FLAG_SHARE_TILES, FLAG_STREAM = 1, 2, 4, 8, 16
 
 
 DFS_ORDER_MAX_NODES = 131072

@@ -191,7 +191,8 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
                   BLOCK_M=128, MAX_ANCESTORS=64, *, out_dtype: Optional[torch.dtype] = None,
                   return_lse: bool = False, fast_pv: bool = False, generic: bool = False,
                   wide_waves: bool = False, key_splits: Optional[int] = None, share_tiles: bool = False,
-                  k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None):
+                  k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None,
+                  stream_blocks: bool = False):
     """Fused sparse tree attention forward (reference ``fstattention.py:153-181``).
 
     ``q [Z,H,Nq,D]``, ``k,v [Z,H,Nk,D]`` (``Nk - Nq`` leading rows are a dense
@@ -210,7 +211,9 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
     results live in a temporary workspace and are joined by a second kernel);
     ``key_splits`` forces the number of runs (``1``: never split); ``share_tiles`` is a tuning
     switch (wave pairs of a row group take alternate key tiles even where the library would let
-    them share the head dimension).  ``k`` and ``v`` may be ``torch.float8_e4m3fn`` (8-bit K/V
+    them share the head dimension); ``stream_blocks`` selects, wherever the shape allows (blocks of 64 or 128
+    rows, head dim 64 or 128, no prefix), the kernel whose workgroups stay and walk a list of query blocks
+    (measured slower than one workgroup per block; kept as a tested alternative).  ``k`` and ``v`` may be ``torch.float8_e4m3fn`` (8-bit K/V
     storage, half the K/V bytes; ``q`` stays float16/bfloat16) with ``k_scale`` / ``v_scale`` float32
     ``[Z*H]`` per-slice scales (``quantize_kv_fp8`` makes all four): the result is that of the 16-bit
     call on ``k * k_scale`` and ``v * v_scale``; block sizes 32/64/128 and head dims 64/128 only, and
@@ -248,10 +251,11 @@ def fst_attention(q, k, v, ancestor_idx, ancestor_mask, leaf_idx, sm_scale,
     if out_code is None:
         raise ValueError("q must be float32/float16/bfloat16 and out_dtype the input dtype or torch.float32")
     flags = 0
-    if fast_pv or generic or wide_waves or key_splits or share_tiles:
+    if fast_pv or generic or wide_waves or key_splits or share_tiles or stream_blocks:
         flags = (_lib.FLAG_FAST_PV if fast_pv else 0) | (_lib.FLAG_GENERIC if generic else 0) | \
             (_lib.FLAG_WIDE_WAVES if wide_waves else 0) | (_lib.flag_key_splits(key_splits) if key_splits else 0) | \
-            (_lib.FLAG_SHARE_TILES if share_tiles else 0)
+            (_lib.FLAG_SHARE_TILES if share_tiles else 0) | \
+            (_lib.FLAG_STREAM if stream_blocks else 0)
     # everything else (the remaining checks, o and L, the workspace of key runs, the launch on the current stream)
     # happens in the registered operator, csrc/fsta_torch_binding.cpp
     o, lse = (_OPS or _ops()).attention_fwd(q, k, v, ancestor_idx, packed.mask_bits, packed.anc_count, leaf_idx, packed.plan,

@@ -198,6 +198,7 @@ extern "C" int fsta_attention_fwd_ws(const void* q, const void* k, const void* v
     p.share_tiles = (flags & FSTA_FLAG_SHARE_TILES) ? 1 : 0;
     p.k_scale = nullptr; p.v_scale = nullptr;
     p.merge_parts = 0; p.dry_run = 0;
+    p.stream_mode = (flags & FSTA_FLAG_STREAM) ? 1 : 0;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (workspace && p.plan) {
@@ -254,8 +255,11 @@ extern "C" int fsta_attention_fwd_ws(const void* q, const void* k, const void* v
         const bool fast_pv = (flags & FSTA_FLAG_FAST_PV) != 0;
         // (the kernel with 16 rows per wave reads the block plan only; it hands launches it cannot
         // take on to the other matrix-core kernel itself)
-        const int rc = (flags & FSTA_FLAG_WIDE_WAVES) || !p.plan ? launch_attention_mfma(p, dtype, head_dim, fast_pv, s)
-                                                                 : launch_attention_mfma16(p, dtype, head_dim, fast_pv, s);
+        int rc = FSTA_EUNSUPPORTED;
+        if (!(flags & FSTA_FLAG_WIDE_WAVES)) rc = launch_attention_stream(p, dtype, head_dim, fast_pv, s);
+        if (rc == FSTA_EUNSUPPORTED)
+            rc = (flags & FSTA_FLAG_WIDE_WAVES) || !p.plan ? launch_attention_mfma(p, dtype, head_dim, fast_pv, s)
+                                                           : launch_attention_mfma16(p, dtype, head_dim, fast_pv, s);
         // ancestor lists too long for the LDS-resident lists of these kernels: the scalar kernel
         // streams them and takes any length
         if (rc != FSTA_EUNSUPPORTED) return rc;
@@ -307,6 +311,6 @@ extern "C" int fsta_attention_fwd_kv8(const void* q, const void* k8, const void*
     p.key_splits = 1; p.split_tiles = 0; p.part_o = nullptr; p.part_lse = nullptr;
     p.share_tiles = 0;
     p.k_scale = k_scale; p.v_scale = v_scale;
-    p.merge_parts = 0; p.dry_run = 0;
+    p.merge_parts = 0; p.dry_run = 0; p.stream_mode = 0;
     return launch_attention_mfma16_kv8(p, dtype, head_dim, static_cast<hipStream_t>(stream));
 }

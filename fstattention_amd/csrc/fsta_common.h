@@ -62,6 +62,7 @@ struct AttnParams {
     // written on the stream) and stores the final rows in o / lse.
     int32_t merge_parts;
     int32_t dry_run;              // launchers return what they would return without launching anything
+    int32_t stream_mode;          // streaming kernel (workgroups that walk a list of blocks): 1 = wherever the shape allows, else never (it is slower than one workgroup per block on every shape measured)
     // 8-bit K/V (fsta_attention_fwd_kv8): k and v hold OCP e4m3 bytes; one float32 scale per
     // (batch, head) slice each, or null for 1
     const float* k_scale;
@@ -120,6 +121,8 @@ int launch_attention_mfma16(const AttnParams& p, int dtype, int head_dim, bool f
 // dense shared prefix, run by run, into slots 1 .. key_splits of p.part_o / p.part_lse
 int launch_attention_prefix(const AttnParams& p, int dtype, int head_dim, bool fast_pv, hipStream_t stream);
 bool prefix_kernel_supported(int dtype, int head_dim);
+// workgroups that stay and walk a list of (block, slice) pairs; FSTA_EUNSUPPORTED where the launch has too few pairs or a prefix
+int launch_attention_stream(const AttnParams& p, int dtype, int head_dim, bool fast_pv, hipStream_t stream);
 int launch_attention_mfma16_kv8(const AttnParams& p, int dtype, int head_dim, hipStream_t stream);
 bool mfma_supported(int dtype, int head_dim, int block_m);
 // joins `splits` partial results (layout of AttnParams::part_o / part_lse) into o (and lse, may be null)

@@ -1,13 +1,15 @@
 """Where a workgroup of the matrix-core attention kernel spends its time.
 
     python -m fstattention_amd.build --timeline        # builds libfsta_timeline.so (-DFSTA_TIMELINE)
-    python -m fstattention_amd.timeline [--config 2] [--warm]
+    python -m fstattention_amd.timeline [--config 2] [--warm] [--stream]
 
 Runs one launch of a benchmark configuration through the instrumented library: every wave notes the
 100 MHz clock at fixed points of the kernel (``FSTA_STAMP`` in ``csrc/fsta_attention_mfma16.hip``)
 (the constant 100 MHz clock, 10 ns per tick).  Printed: the mean time between consecutive points over all
 waves, a wave's lifetime and the spread of the waves' start times.  Every stamp is a scalar memory
-instruction the wave waits for: the shares matter, not the total.  Measuring tool; the regular library has no such code.
+instruction the wave waits for: the shares matter, not the total.  ``--stream`` runs the streaming kernel (``csrc/fsta_attention_stream.hip``, workgroups that walk a list of blocks)
+instead and prints where its waves' shader-clock cycles go, by kind of segment.
+Measuring tool; the regular library has no such code.
 """
 from __future__ import annotations
 
@@ -34,6 +36,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--config", type=int, default=2)
     ap.add_argument("--warm", action="store_true", help="run the launch twice on the same buffers and time the second")
+    ap.add_argument("--stream", action="store_true", help="the streaming kernel's cycle shares instead")
     args = ap.parse_args()
     if not os.path.exists(TIMELINE_LIB_PATH):
         raise SystemExit(f"{TIMELINE_LIB_PATH} is missing: python -m fstattention_amd.build --timeline")
@@ -59,12 +62,16 @@ def main():
     # flush the caches with a large fill so that q/k/v come from HBM, unless a warm run is wanted
     flush = torch.empty((1 << 30,), dtype=torch.uint8, device=dev)
 
-    def launch():
+    def launch(flags=0):
         rc = fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), None, a_idx.data_ptr(), packed.mask_bits.data_ptr(),
                  packed.anc_count.data_ptr(), l_idx.data_ptr(), packed.plan.data_ptr(), 0, cfg.batch, cfg.heads, cfg.n_nodes,
                  cfg.n_nodes, cfg.head_dim, code, code, cfg.block_m, max_anc, a_idx.shape[0], 1.0 / math.sqrt(cfg.head_dim),
-                 0, torch.cuda.current_stream().cuda_stream)
+                 flags, torch.cuda.current_stream().cuda_stream)
         assert rc == 0, lib.fsta_last_error()
+
+    if args.stream:
+        stream_shares(lib, launch, flush, cfg)
+        return
 
     assert lib.fsta_timeline_buffer(None) == 0
     launch()                                   # first launch: code upload, LDS limits
@@ -98,6 +105,37 @@ def main():
     start = (real[:, 0] - real[:, 0].min()) / 100.0
     end = (real[:, 1] - real[:, 0].min()) / 100.0
     print(f"waves start over {start.max():.2f} us (mean {start.mean():.2f}); the last one ends {end.max():.2f} us after the first started")
+
+
+SEGMENTS = ["wait for the step's tile (vmcnt)", "workgroup barrier", "plan published, next tile requested (scalar bookkeeping)",
+            "Q fragments read", "leaf tile, own rows", "leaf tile, other waves' rows", "ancestor tile computed",
+            "ancestor tile skipped (no query of the wave attends)", "normalise, store, next pair"]
+
+
+def stream_shares(lib, launch, flush, cfg):
+    """One launch of the streaming kernel: cycles per kind of segment, summed per wave by the kernel itself."""
+    lib.fsta_stream_profile_buffer.restype, lib.fsta_stream_profile_buffer.argtypes = ctypes.c_int, [ctypes.c_void_p]
+    waves = cfg.block_m // 16
+    buf = torch.zeros((512 * waves * 20,), dtype=torch.int64, device=flush.device)
+    assert lib.fsta_stream_profile_buffer(None) == 0
+    launch(_lib.FLAG_STREAM)
+    flush.fill_(1)
+    torch.cuda.synchronize()
+    assert lib.fsta_stream_profile_buffer(buf.data_ptr()) == 0
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    launch(_lib.FLAG_STREAM)
+    ev1.record()
+    torch.cuda.synchronize()
+    print(f"kernel: {lib.fsta_last_attention_kernel().decode()} (instrumented), {ev0.elapsed_time(ev1) * 1e3:.1f} us")
+    data = buf.cpu().numpy().reshape(-1, 20)
+    data = data[data[:, 10:].sum(1) != 0]
+    cyc, cnt = data[:, :10].sum(0), data[:, 10:].sum(0)
+    n = data.shape[0]
+    print(f"workload: {cfg.name}; {n} waves; shader-clock cycles per wave: {cyc.sum() / n:.0f}")
+    print(f"{'segment':<60}{'share':>8}{'times per wave':>16}{'cycles each':>14}")
+    for i, name in enumerate(SEGMENTS):
+        print(f"{name:<60}{100.0 * cyc[i] / cyc.sum():>7.1f}%{cnt[i] / n:>16.1f}{cyc[i] / max(cnt[i], 1):>14.0f}")
 
 
 if __name__ == "__main__":

@@ -47,6 +47,11 @@ extern "C" {
 #define FSTA_FLAG_SHARE_TILES 8u /* tuning: where two waves share a group of 16 query rows they
                                   always take alternate key tiles (and merge at the end), never
                                   halves of the head dimension                              */
+#define FSTA_FLAG_STREAM 16u    /* tuning/tests: workgroups that stay and walk a list of query blocks
+                                  * (the streaming kernel, one launch of as many workgroups as the GPU
+                                  * holds) wherever the shape allows: block_m 64/128, head_dim 64/128,
+                                  * 16-bit types, no prefix, a block plan.  Measured slower than one
+                                  * workgroup per block, so the library never takes it by itself. */
 #define FSTA_FLAG_KEY_SPLITS(n) (((uint32_t)(n) & 0xffu) << 8)
                                /* fsta_attention_fwd_ws / fsta_attention_workspace_bytes:
                                   cut the shared prefix into n runs of keys (n = 1: never

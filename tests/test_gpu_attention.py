@@ -21,7 +21,8 @@ pytestmark = pytest.mark.gpu
 
 
 def run_tree(parent, block_m, z, h, d, dtype, seed, prefix=0, generic=False, fast_pv=False,
-             scale=None, check_lse=True, wide_waves=False, key_splits=None, share_tiles=False):
+             scale=None, check_lse=True, wide_waves=False, key_splits=None, share_tiles=False, stream_blocks=None,
+             native_out=False, want_kernel=None):
     n = len(parent)
     a_idx, a_mask, l_idx, max_anc = oracle_inputs(parent, block_m)
     nb = a_idx.shape[0]
@@ -34,7 +35,18 @@ def run_tree(parent, block_m, z, h, d, dtype, seed, prefix=0, generic=False, fas
     o, lse = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(),
                            scale, BLOCK_M=block_m, MAX_ANCESTORS=max_anc,
                            out_dtype=torch.float32, return_lse=True, generic=generic, fast_pv=fast_pv,
-                           wide_waves=wide_waves, key_splits=key_splits, share_tiles=share_tiles)
+                           wide_waves=wide_waves, key_splits=key_splits, share_tiles=share_tiles,
+                           stream_blocks=stream_blocks)
+    if want_kernel is not None:
+        from fstattention_amd import _lib
+        assert want_kernel in _lib.load().fsta_last_attention_kernel().decode()
+    if native_out:      # the output in the type of q: within one unit in the last place of the float32 result
+        o_native = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(), scale,
+                                 BLOCK_M=block_m, MAX_ANCESTORS=max_anc, generic=generic, fast_pv=fast_pv,
+                                 wide_waves=wide_waves, key_splits=key_splits, share_tiles=share_tiles,
+                                 stream_blocks=stream_blocks)
+        assert o_native.dtype == dtype
+        torch.testing.assert_close(o_native.float(), o.to(dtype).float(), atol=0, rtol=2 ** -7 if dtype == torch.bfloat16 else 2 ** -10)
     assert o.dtype == torch.float32 and o.shape == q.shape
     err = assert_close(o, want, dtype, f"n={n} m={block_m} d={d} {dtype} prefix={prefix}")
     if check_lse:
