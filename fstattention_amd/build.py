@@ -43,7 +43,7 @@ HIPCC_FLAGS = [
 # Kernels of these sources must keep everything in registers: a private array the compiler leaves
 # in scratch memory, or a spill, is reloaded through the same vmcnt queue their gather rings count on.
 NO_SCRATCH = ("fsta_attention_mfma16.hip", "fsta_attention_mfma.hip", "fsta_attention_prefix.hip",
-              "fsta_attention_stream.hip")
+              "fsta_attention_stream.hip", "fsta_attention_generic.hip")
 
 
 def _hipcc() -> str:

@@ -66,16 +66,6 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
     const T* vb = static_cast<const T*>(p.v) + (size_t)hz * p.nk * D;
 
     constexpr int kVec = Vec16<T>::n;           // elements per 16-byte global load
-    for (int e = tid; e < M * D / kVec; e += kThreads) {
-        const int m = e / (D / kVec), d = (e % (D / kVec)) * kVec;
-        const int row = row0 + m;
-        float x[kVec];
-#pragma unroll
-        for (int i = 0; i < kVec; ++i) x[i] = 0.f;
-        if (row < p.nq) load16(qb + (size_t)row * D + d, x);
-#pragma unroll
-        for (int i = 0; i < kVec; ++i) q_s[m * kPitch + d + i] = x[i];
-    }
 
     // this thread's tiles
     const int sc = (tid % kColGroupsS) * 4;     // first key column of the score tile
@@ -87,8 +77,20 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
     for (int i = 0; i < kRowsO; ++i)
 #pragma unroll
         for (int c = 0; c < 4; ++c) acc[i][c] = 0.f;
-    float m_i = -INFINITY, l_i = 0.f;  // running max / sum of row `tid` (tid < M)
+    // running maximum / sum of this thread's score rows (the 8 threads that share a row hold the same values)
+    float m_i[kRowsS], l_i[kRowsS];
+#pragma unroll
+    for (int i = 0; i < kRowsS; ++i) { m_i[i] = -INFINITY; l_i[i] = 0.f; }
 
+    // the block's ancestor count and the first entries of both lists are requested together: which of the
+    // two lists tile 0 (and tile 1) comes from depends on the count, and the count is one more round trip
+    int64_t first_anc0 = -1, first_anc1 = -1, first_leaf0 = -1, first_leaf1 = -1;
+    if (tid < kTileN) {
+        if (tid < p.max_anc) first_anc0 = p.ancestor_idx[(size_t)j * p.max_anc + tid];
+        if (kTileN + tid < p.max_anc) first_anc1 = p.ancestor_idx[(size_t)j * p.max_anc + kTileN + tid];
+        if (tid < M) first_leaf0 = p.leaf_idx[(size_t)j * M + tid];
+        if (kTileN + tid < M) first_leaf1 = p.leaf_idx[(size_t)j * M + kTileN + tid];
+    }
     int n_anc = p.anc_count ? p.anc_count[j] : p.max_anc;
     n_anc = min(max(n_anc, 0), p.max_anc);
     const int anc_tiles = (n_anc + kTileN - 1) / kTileN;
@@ -136,11 +138,42 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
         }
     };
     if (tid < kTileN) {
-        key_s[tid] = load_key(0);
-        key_s[kTileN + tid] = load_key(1);
+        // tiles 0 and 1 from the entries requested above where they are ancestor or leaf tiles
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            int key = -1;
+            if (t < total_tiles) {
+                int base;
+                const int kind = tile_kind(t, base);
+                if (kind == 2 || base >= 2 * kTileN) {
+                    key = load_key(t);
+                } else {
+                    const int c = base + tid;
+                    // (unary plus: a choice between values, not between addresses)
+                    const int64_t from_anc = base == 0 ? +first_anc0 : +first_anc1;
+                    const int64_t from_leaf = base == 0 ? +first_leaf0 : +first_leaf1;
+                    const int64_t idx = kind == 0 ? (c < n_anc ? from_anc : -1) : (c < M ? from_leaf : -1);
+                    key = (idx >= 0 && idx < p.nk) ? (int)idx : -1;
+                }
+            }
+            key_s[t * kTileN + tid] = key;
+        }
     }
     __syncthreads();
     if (total_tiles > 0) fetch_rows(key_s);
+    // The Q rows are requested behind the first tile's K/V rows (both are needed at the same moment, the first
+    // score tile): in front of the key lists they would put one more memory round trip into the start-up chain.
+    for (int e = tid; e < M * D / kVec; e += kThreads) {
+        const int m = e / (D / kVec), d = (e % (D / kVec)) * kVec;
+        const int row = row0 + m;
+        float x[kVec];
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) x[i] = 0.f;
+        if (row < p.nq) load16(qb + (size_t)row * D + d, x);
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) q_s[m * kPitch + d + i] = x[i];
+    }
+
 
     for (int t = 0; t < total_tiles; ++t) {
         int base;
@@ -171,52 +204,77 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
             for (int i = 0; i < kRowsS; ++i)
 #pragma unroll
                 for (int c = 0; c < 4; ++c) dot[i][c] = 0.f;
-#pragma unroll 4
-            for (int d = 0; d < D; d += 4) {
-                float4 kq[4];
-#pragma unroll
-                for (int c = 0; c < 4; ++c) kq[c] = *reinterpret_cast<const float4*>(k_s + (sc + c) * kPitch + d);
+            if (kind == 1) {
+                // leaf tile: row m sees its own key only (column m - base): one dot product per row, by the thread
+                // whose four columns hold it
 #pragma unroll
                 for (int i = 0; i < kRowsS; ++i) {
                     const int m = sr + kRowSlotsS * i;
-                    if (kRowsS * kRowSlotsS > M && m >= M) continue;
-                    const float4 qq = *reinterpret_cast<const float4*>(q_s + m * kPitch + d);
+                    const int own = m - base - sc;
+                    if ((kRowsS * kRowSlotsS > M && m >= M) || own < 0 || own >= 4) continue;
+                    float part = 0.f;
+#pragma unroll 4
+                    for (int d = 0; d < D; d += 4) {
+                        const float4 kk = *reinterpret_cast<const float4*>(k_s + (sc + own) * kPitch + d);
+                        const float4 qq = *reinterpret_cast<const float4*>(q_s + m * kPitch + d);
+                        part += qq.x * kk.x + qq.y * kk.y + qq.z * kk.z + qq.w * kk.w;
+                    }
 #pragma unroll
-                    for (int c = 0; c < 4; ++c)
-                        dot[i][c] += qq.x * kq[c].x + qq.y * kq[c].y + qq.z * kq[c].z + qq.w * kq[c].w;
+                    for (int c = 0; c < 4; ++c) dot[i][c] = c == own ? part : dot[i][c];
+                }
+            } else {
+#pragma unroll 4
+                for (int d = 0; d < D; d += 4) {
+                    float4 kq[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) kq[c] = *reinterpret_cast<const float4*>(k_s + (sc + c) * kPitch + d);
+#pragma unroll
+                    for (int i = 0; i < kRowsS; ++i) {
+                        const int m = sr + kRowSlotsS * i;
+                        if (kRowsS * kRowSlotsS > M && m >= M) continue;
+                        const float4 qq = *reinterpret_cast<const float4*>(q_s + m * kPitch + d);
+#pragma unroll
+                        for (int c = 0; c < 4; ++c)
+                            dot[i][c] += qq.x * kq[c].x + qq.y * kq[c].y + qq.z * kq[c].z + qq.w * kq[c].w;
+                    }
                 }
             }
+            // mask, then the online softmax of the row among the 8 threads that share it (neighbouring lanes:
+            // maximum and sum by lane exchanges), weights into s_s for the O tiles
 #pragma unroll
             for (int i = 0; i < kRowsS; ++i) {
                 const int m = sr + kRowSlotsS * i;
-                if (kRowsS * kRowSlotsS > M && m >= M) continue;
+                if (kRowsS * kRowSlotsS > M && m >= M) continue;     // (whole waves: M is a multiple of 16, a wave holds 8 rows)
                 uint32_t w = 0xffffffffu;
                 if (kind == 0) w = p.mask_bits[((size_t)j * p.mask_words + (base >> 5)) * M + m];
+                float sv[4];
+                float mx = -INFINITY;
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     const int n = sc + c;
                     bool ok = keys[n] >= 0 && ((w >> n) & 1u);
                     if (kind == 1) ok = ok && (m == base + n);
-                    s_s[m * kPitchS + n] = ok ? dot[i][c] * p.scale_log2e : -INFINITY;
+                    sv[c] = ok ? dot[i][c] * p.scale_log2e : -INFINITY;
+                    mx = fmaxf(mx, sv[c]);
                 }
+#pragma unroll
+                for (int dlt = 1; dlt < kColGroupsS; dlt <<= 1) mx = fmaxf(mx, __shfl_xor(mx, dlt));
+                const float m_new = fmaxf(m_i[i], mx);
+                const float alpha = (m_new == -INFINITY) ? 1.f : exp2f(m_i[i] - m_new);
+                float sum = 0.f;
+                float wv[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    wv[c] = (sv[c] == -INFINITY) ? 0.f : exp2f(sv[c] - m_new);
+                    sum += wv[c];
+                }
+                *reinterpret_cast<float4*>(s_s + m * kPitchS + sc) = make_float4(wv[0], wv[1], wv[2], wv[3]);
+#pragma unroll
+                for (int dlt = 1; dlt < kColGroupsS; dlt <<= 1) sum += __shfl_xor(sum, dlt);
+                l_i[i] = l_i[i] * alpha + sum;
+                m_i[i] = m_new;
+                if (sc == 0) alpha_s[m] = alpha;
             }
-        }
-        __syncthreads();
-
-        if (tid < M) {
-            float mx = m_i;
-            for (int n = 0; n < kTileN; ++n) mx = fmaxf(mx, s_s[tid * kPitchS + n]);
-            const float alpha = (mx == -INFINITY) ? 1.f : exp2f(m_i - mx);
-            float sum = 0.f;
-            for (int n = 0; n < kTileN; ++n) {
-                const float s = s_s[tid * kPitchS + n];
-                const float w = (s == -INFINITY) ? 0.f : exp2f(s - mx);
-                s_s[tid * kPitchS + n] = w;
-                sum += w;
-            }
-            l_i = l_i * alpha + sum;
-            m_i = mx;
-            alpha_s[tid] = alpha;
         }
         __syncthreads();
 
@@ -230,20 +288,36 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
 #pragma unroll
                 for (int c = 0; c < 4; ++c) acc[i][c] *= a;
             }
-#pragma unroll 2
-            for (int n = 0; n < kTileN; n += 4) {
-                float4 vv[4];
-#pragma unroll
-                for (int u = 0; u < 4; ++u) vv[u] = *reinterpret_cast<const float4*>(v_s + (n + u) * kPitch + oc);
+            if (kind == 1) {
+                // leaf tile: a row's only weight sits on its own key
 #pragma unroll
                 for (int i = 0; i < kRowsO; ++i) {
                     const int m = orow + kRowSlotsO * i;
-                    if (kRowsO * kRowSlotsO > M && m >= M) continue;
-                    const float4 w = *reinterpret_cast<const float4*>(s_s + m * kPitchS + n);
-                    acc[i][0] += w.x * vv[0].x + w.y * vv[1].x + w.z * vv[2].x + w.w * vv[3].x;
-                    acc[i][1] += w.x * vv[0].y + w.y * vv[1].y + w.z * vv[2].y + w.w * vv[3].y;
-                    acc[i][2] += w.x * vv[0].z + w.y * vv[1].z + w.z * vv[2].z + w.w * vv[3].z;
-                    acc[i][3] += w.x * vv[0].w + w.y * vv[1].w + w.z * vv[2].w + w.w * vv[3].w;
+                    const int own = m - base;
+                    if ((kRowsO * kRowSlotsO > M && m >= M) || own < 0 || own >= kTileN) continue;
+                    const float w = s_s[m * kPitchS + own];
+                    const float4 vv = *reinterpret_cast<const float4*>(v_s + own * kPitch + oc);
+                    acc[i][0] += w * vv.x;
+                    acc[i][1] += w * vv.y;
+                    acc[i][2] += w * vv.z;
+                    acc[i][3] += w * vv.w;
+                }
+            } else {
+#pragma unroll 2
+                for (int n = 0; n < kTileN; n += 4) {
+                    float4 vv[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) vv[u] = *reinterpret_cast<const float4*>(v_s + (n + u) * kPitch + oc);
+#pragma unroll
+                    for (int i = 0; i < kRowsO; ++i) {
+                        const int m = orow + kRowSlotsO * i;
+                        if (kRowsO * kRowSlotsO > M && m >= M) continue;
+                        const float4 w = *reinterpret_cast<const float4*>(s_s + m * kPitchS + n);
+                        acc[i][0] += w.x * vv[0].x + w.y * vv[1].x + w.z * vv[2].x + w.w * vv[3].x;
+                        acc[i][1] += w.x * vv[0].y + w.y * vv[1].y + w.z * vv[2].y + w.w * vv[3].y;
+                        acc[i][2] += w.x * vv[0].z + w.y * vv[1].z + w.z * vv[2].z + w.w * vv[3].z;
+                        acc[i][3] += w.x * vv[0].w + w.y * vv[1].w + w.z * vv[2].w + w.w * vv[3].w;
+                    }
                 }
             }
         }
@@ -251,11 +325,16 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
         __syncthreads();
     }
 
-    if (tid < M) {
-        stat_s[tid] = l_i;
-        const int row = row0 + tid;
-        if (p.lse && row < p.nq)
-            p.lse[(size_t)hz * p.nq + row] = l_i > 0.f ? m_i + log2f(l_i) : -INFINITY;
+    if (sr < M && sc == 0) {
+#pragma unroll
+        for (int i = 0; i < kRowsS; ++i) {
+            const int m = sr + kRowSlotsS * i;
+            if (kRowsS * kRowSlotsS > M && m >= M) continue;
+            stat_s[m] = l_i[i];
+            const int row = row0 + m;
+            if (p.lse && row < p.nq)
+                p.lse[(size_t)hz * p.nq + row] = l_i[i] > 0.f ? m_i[i] + log2f(l_i[i]) : -INFINITY;
+        }
     }
     __syncthreads();
 
