@@ -316,8 +316,8 @@ def time_front_end(index, reps=20, stages=None):
     draft probabilities -> parent array (cfg2's generator only), depth-first order, parent array ->
     lineage, lineage -> kernel inputs."""
     import torch
-    from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, lineage_from_parents_gpu,
-                                  medusa_parents_gpu, trees)
+    from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, kernel_inputs_from_parents_gpu,
+                                  lineage_from_parents_gpu, medusa_parents_gpu, trees)
     dev = torch.device("cuda", 0)
     cfg = trees.config(index)
     parent = torch.from_numpy(cfg.parent).to(dev)
@@ -350,6 +350,8 @@ def time_front_end(index, reps=20, stages=None):
         "lineage_from_parents_us": lambda: lineage_from_parents_gpu(parent, width=width, check=False),
         "kernel_inputs_us": lambda: create_fst_attention_kernel_inputs(
             lineage, level, cfg.block_m, max_anc, mutate_lineage=False, check=False, want_bool_mask=False),
+        # the two stages above in one launch (lineage rows built in every workgroup's LDS)
+        "kernel_inputs_from_parents_us": lambda: kernel_inputs_from_parents_gpu(parent, cfg.block_m, max_anc, width, check=False),
     }
     if index == 2:
         probs = torch.from_numpy(trees.medusa_probs()).to(dev)
@@ -360,12 +362,13 @@ def time_front_end(index, reps=20, stages=None):
     return {name: device_us(fn) for name, fn in calls.items() if stages is None or name in stages}
 
 
-def time_decoding_step(wl, layers=32, reps=5, depth_first=True):
+def time_decoding_step(wl, layers=32, reps=5, depth_first=True, fused=True):
     """One decoding step of the headline workload as one HIP graph: draft probabilities -> tree ->
-    (depth-first order ->) lineage -> kernel inputs (once), then `layers` attention calls on rotating
+    (depth-first order ->) kernel inputs (lineage rows built inside that launch; `fused=False`: lineage and kernel inputs as
+    two launches) once, then `layers` attention calls on rotating
     q/k/v/o sets that all use those inputs.  Microseconds per step from HIP events."""
     import torch
-    from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, fst_attention,
+    from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, fst_attention, kernel_inputs_from_parents_gpu,
                                   lineage_from_parents_gpu, medusa_parents_gpu, renumber_parents_gpu, trees)
     dev = torch.device("cuda", 0)
     probs = torch.from_numpy(trees.medusa_probs()).to(dev)
@@ -377,9 +380,12 @@ def time_decoding_step(wl, layers=32, reps=5, depth_first=True):
         if depth_first:
             perm, rank = dfs_order_gpu(parent, "light_first", check=False, status=status)
             parent = renumber_parents_gpu(parent, perm, rank)
-        lineage, level = lineage_from_parents_gpu(parent, width=depths + 1, check=False, status=status)
-        a_idx, packed, l_idx, _ = create_fst_attention_kernel_inputs(
-            lineage, level, wl.m, wl.max_anc, check=False, want_bool_mask=False, status=status)
+        if fused:
+            a_idx, packed, l_idx, _ = kernel_inputs_from_parents_gpu(parent, wl.m, wl.max_anc, depths + 1, check=False, status=status)
+        else:
+            lineage, level = lineage_from_parents_gpu(parent, width=depths + 1, check=False, status=status)
+            a_idx, packed, l_idx, _ = create_fst_attention_kernel_inputs(
+                lineage, level, wl.m, wl.max_anc, check=False, want_bool_mask=False, status=status)
         for layer in range(layers):
             q, k, v, _ = wl.sets[layer % wl.n_sets]
             fst_attention(q, k, v, a_idx, packed, l_idx, wl.scale, BLOCK_M=wl.m, MAX_ANCESTORS=wl.max_anc)
@@ -802,6 +808,18 @@ def main():
         result["configs"] = other_configurations(use_graph, wl)
         result["reference_benchmark"] = reference_benchmark(use_graph)
         result["fp8_kv_storage"] = fp8_kv_storage(use_graph)
+        if headline:
+            # the integer kernels that turn a new tree into kernel inputs once per decoding step, and the whole step
+            result["front_end_device_us"] = {"cfg2_medusa256": time_front_end(2)}
+            result["cfg2_decoding_step"] = {
+                "layers": 32,
+                "total_us": round(time_decoding_step(wl, depth_first=False), 1),
+                "total_us_lineage_and_kernel_inputs_as_two_launches": round(time_decoding_step(wl, depth_first=False, fused=False), 1),
+                "total_us_depth_first_order": round(time_decoding_step(wl), 1),
+                "note": "one graph: probabilities -> tree (-> depth-first order) -> lineage -> kernel inputs, then 32 "
+                        "attention calls (Python wrapper, output allocated per call) on rotating q/k/v sets; a tree "
+                        "this small gains nothing from the depth-first order, the large ones do",
+            }
     if args.extra:
         extra = {}
         for idx in (3, 4, 5):
@@ -855,18 +873,9 @@ def main():
             }
             del w
             torch.cuda.empty_cache()
-        extra["cfg2_decoding_step"] = {
-            "layers": 32,
-            "total_us": round(time_decoding_step(wl, depth_first=False), 1),
-            "total_us_depth_first_order": round(time_decoding_step(wl), 1),
-            "note": "one graph: probabilities -> tree (-> depth-first order) -> lineage -> kernel inputs, then 32 "
-                    "attention calls (Python wrapper, output allocated per call) on rotating q/k/v sets; a tree "
-                    "this small gains nothing from the depth-first order, the large ones do",
-        }
         # the integer kernels that turn a new tree into kernel inputs once per decoding step
         extra["front_end_device_us"] = {trees_name: time_front_end(idx) for idx, trees_name in
-                                        ((2, "cfg2_medusa256"), (3, "cfg3_deep1024"), (4, "cfg4_wide4096"),
-                                         (5, "cfg5_batched2048"))}
+                                        ((3, "cfg3_deep1024"), (4, "cfg4_wide4096"), (5, "cfg5_batched2048"))}
         # the headline tree behind a shared prefix (the KV cache of a decoding step, reference
         # fstattention.py:113-136): the prefix as each block's own loop, and cut into runs of keys
         for prefix in (4096, 16384):

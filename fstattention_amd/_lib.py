@@ -39,6 +39,8 @@ SIGNATURES = {
     "fsta_block_plan_bytes": (c_size_t, [c_int32, c_int32, c_int32]),
     "fsta_precompute": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int32, c_int32,
                                 c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "fsta_precompute_from_parents": (c_int, [c_void_p, c_int64, c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p,
+                                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "fsta_pack_mask": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int64, c_void_p, c_void_p,
                                c_void_p, c_void_p]),
     "fsta_attention_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,

@@ -26,7 +26,11 @@ __global__ __launch_bounds__(kMaxThreads) void block_precompute_kernel(
     int64_t n_nodes, int64_t width, int block_m, int max_anc, int mask_words, int mutate, int staged,
     int64_t* __restrict__ ancestor_idx, uint8_t* __restrict__ ancestor_mask,
     int64_t* __restrict__ leaf_idx, uint32_t* __restrict__ mask_bits,
-    int32_t* __restrict__ anc_count, uint32_t* __restrict__ plan, uint32_t* __restrict__ status) {
+    int32_t* __restrict__ anc_count, uint32_t* __restrict__ plan, const int64_t* __restrict__ parent,
+    uint32_t* __restrict__ status) {
+    // `parent` != NULL (fsta_precompute_from_parents): the block's lineage rows are not read but built here, from the
+    // parent array (copied into LDS as int32 behind the staged rows); `lineage` and `level_lookup` are then outputs
+    // (each may be NULL) and `staged` is 1.
     extern __shared__ uint32_t lds[];
     const int n_words = (int)((n_nodes + 31) >> 5);
     uint32_t* bitmap = lds;                                   // ancestor set of this block
@@ -54,13 +58,53 @@ __global__ __launch_bounds__(kMaxThreads) void block_precompute_kernel(
         }
     };
     int64_t first[kBatch];
-    load_batch(tid, first);
+    if (!parent) load_batch(tid, first);
+    int32_t* par_s = vals_s + (size_t)block_m * width;      // [n_nodes], from-parents mode only
+    uint32_t err = 0u;
+    if (parent) {
+        for (int64_t i = tid; i < n_nodes; i += threads) {
+            const int64_t pp = parent[i];
+            const bool ok = pp >= -1 && pp < i;
+            if (!ok) err |= FSTA_PRE_BAD_NODE_ID;
+            par_s[i] = ok ? (int32_t)pp : -1;
+        }
+    }
 
     for (int w = tid; w < n_words; w += threads) bitmap[w] = 0u;
     for (int e = tid; e < mask_words * block_m; e += threads) mbits[e] = 0u;
     if (tid < 4) misc[tid] = 0u;
-    uint32_t err = 0u;
-    for (int r = tid; r < block_m; r += threads) {
+    if (parent) {
+        __syncthreads();
+        // One lane per row walks to the root once and notes the ancestors in hop order (every hop goes to a smaller
+        // id, so the walk ends), then turns its row around into level order, -1 padded (layout of utils.py:66-75:
+        // column l = the ancestor at level l; the node's own column holds -1 until the self entry goes in).
+        for (int r = tid; r < block_m; r += threads) {
+            int32_t lv = -1;
+            if (r < rows) {
+                int32_t* row = vals_s + (size_t)r * width;
+                int32_t depth = 0;
+                for (int32_t a = par_s[lo + r]; a >= 0; a = par_s[a]) {
+                    if (depth < width) row[depth] = a;
+                    ++depth;
+                }
+                if (depth >= width) {          // deeper than the rows are wide: flagged, the row counts as empty
+                    err |= FSTA_PRE_BAD_LEVEL;
+                    depth = 0;
+                } else {
+                    lv = depth;
+                }
+                for (int32_t a = 0, b = depth - 1; a < b; ++a, --b) {
+                    const int32_t x = row[a];
+                    row[a] = row[b];
+                    row[b] = x;
+                }
+                for (int32_t l = depth; l < width; ++l) row[l] = -1;
+                if (level_lookup) const_cast<int64_t*>(level_lookup)[lo + r] = lv >= 0 ? lv : 0;
+            }
+            lvl_s[r] = lv;
+        }
+    }
+    for (int r = tid; r < block_m && !parent; r += threads) {
         int32_t lv = -1;  // -1 = nothing to insert (pad row or invalid level)
         if (r < rows) {
             int64_t l = level_lookup[lo + r];
@@ -93,11 +137,27 @@ __global__ __launch_bounds__(kMaxThreads) void block_precompute_kernel(
             if (staged) vals_s[e] = keep;
         }
     };
+    if (parent) {
+        __syncthreads();      // the rows are complete
+        for (uint32_t e = tid; e < n_elem; e += threads) {
+            const int32_t v = vals_s[e];
+            if (v < 0) saw_pad = true;
+            else {
+                const uint32_t bit = 1u << (v & 31);
+                if (!(bitmap[v >> 5] & bit)) atomicOr(&bitmap[v >> 5], bit);
+            }
+            if (lineage) {      // the rows as the lineage tensor (with the self entries when asked for)
+                const uint32_t r = e / (uint32_t)width, l = e - r * (uint32_t)width;
+                lineage[lo * width + e] = (mutate && (int32_t)l == lvl_s[r]) ? lo + r : (int64_t)v;
+            }
+        }
+    } else {
     take_batch(tid, first);
     for (uint32_t e0 = tid + (uint32_t)threads * kBatch; e0 < n_elem; e0 += (uint32_t)threads * kBatch) {
         int64_t val[kBatch];
         load_batch(e0, val);
         take_batch(e0, val);
+    }
     }
     if (saw_pad) misc[0] = 1u;
     __syncthreads();
@@ -253,7 +313,7 @@ __global__ __launch_bounds__(kMaxThreads) void block_precompute_kernel(
     }
 
     // 6. the caller's lineage receives the self entries (utils.py:118,125)
-    if (mutate) {
+    if (mutate && !parent) {
         for (int r = tid; r < rows; r += threads)
             if (lvl_s[r] >= 0) lineage[(lo + r) * width + lvl_s[r]] = lo + r;
     }
@@ -472,7 +532,48 @@ extern "C" int fsta_precompute(int64_t* lineage, const int64_t* level_lookup, in
     hipLaunchKernelGGL(block_precompute_kernel, dim3((unsigned)nb), dim3(threads), lds,
                        static_cast<hipStream_t>(stream), lineage, level_lookup, n_nodes, width,
                        block_m, max_ancestors, mask_words, mutate_lineage, staged, ancestor_idx,
-                       ancestor_mask, leaf_idx, mask_bits, anc_count, block_plan, status);
+                       ancestor_mask, leaf_idx, mask_bits, anc_count, block_plan, nullptr, status);
+    FSTA_HIP_OK(hipGetLastError());
+    return FSTA_OK;
+}
+
+extern "C" int fsta_precompute_from_parents(const int64_t* parent, int64_t n_nodes, int64_t width, int32_t block_m,
+                                            int32_t max_ancestors, int32_t insert_self, int64_t* lineage,
+                                            int64_t* level_lookup, int64_t* ancestor_idx, uint8_t* ancestor_mask,
+                                            int64_t* leaf_idx, uint32_t* mask_bits, int32_t* anc_count,
+                                            uint32_t* block_plan, uint32_t* status, void* stream) {
+    if (n_nodes < 0 || width < 1 || block_m < 1 || max_ancestors < 1)
+        return fail(FSTA_EINVAL, "fsta_precompute_from_parents: n_nodes=%lld width=%lld block_m=%d max_ancestors=%d",
+                    (long long)n_nodes, (long long)width, block_m, max_ancestors);
+    if (n_nodes == 0) return FSTA_OK;
+    if (!parent || !ancestor_idx || !leaf_idx || !status) return fail(FSTA_EINVAL, "fsta_precompute_from_parents: null pointer");
+    if (block_m > 4096) return fail(FSTA_EUNSUPPORTED, "fsta_precompute_from_parents: block_m=%d > 4096", block_m);
+    if (block_plan && !plan_block_size_ok(block_m))
+        return fail(FSTA_EINVAL, "fsta_precompute_from_parents: a block plan needs block_m 32, 64 or 128 (got %d)", block_m);
+    if (misaligned(parent, 8) || misaligned(lineage, 8) || misaligned(level_lookup, 8) || misaligned(ancestor_idx, 8) ||
+        misaligned(leaf_idx, 8))
+        return fail(FSTA_EINVAL, "fsta_precompute_from_parents: parent, lineage, level_lookup, ancestor_idx and leaf_idx must be 8-byte aligned");
+    if (misaligned(mask_bits, 4) || misaligned(anc_count, 4) || misaligned(status, 4) || misaligned(block_plan, 16))
+        return fail(FSTA_EINVAL, "fsta_precompute_from_parents: mask_bits, anc_count and status must be 4-byte aligned, block_plan 16-byte");
+    const int mask_words = fsta_mask_words(max_ancestors);
+    const int64_t n_words = (n_nodes + 31) >> 5;
+    // tables, the block's rows and the parent array, all in one workgroup's LDS
+    const double need = 4.0 * ((double)precompute_lds_words(n_words, mask_words, block_m) + (double)block_m * (double)width + (double)n_nodes);
+    if (need > 160.0 * 1024)
+        return fail(FSTA_EUNSUPPORTED, "fsta_precompute_from_parents: n_nodes=%lld width=%lld block_m=%d max_ancestors=%d need %.0f "
+                    "bytes of LDS (limit 163840): fsta_lineage_from_parents + fsta_precompute take any size",
+                    (long long)n_nodes, (long long)width, block_m, max_ancestors, need);
+    const size_t lds = (size_t)need;
+    if (lds > 64 * 1024) {
+        const int rc = allow_full_lds<&block_precompute_kernel>();
+        if (rc != FSTA_OK) return rc;
+    }
+    const int64_t nb = (n_nodes + block_m - 1) / block_m;
+    const size_t entries = (size_t)block_m * (size_t)width;
+    const int threads = entries >= 2048 || (size_t)block_m * max_ancestors >= 8192 || n_nodes >= 2048 ? kMaxThreads : kThreads;
+    hipLaunchKernelGGL(block_precompute_kernel, dim3((unsigned)nb), dim3(threads), lds, static_cast<hipStream_t>(stream), lineage,
+                       level_lookup, n_nodes, width, block_m, max_ancestors, mask_words, insert_self ? 1 : 0, 1, ancestor_idx,
+                       ancestor_mask, leaf_idx, mask_bits, anc_count, block_plan, parent, status);
     FSTA_HIP_OK(hipGetLastError());
     return FSTA_OK;
 }

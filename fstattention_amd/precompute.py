@@ -85,6 +85,59 @@ def create_fst_attention_kernel_inputs(lineage, level_lookup, block_m=64, max_an
     return out if check else out + (status,)
 
 
+def kernel_inputs_from_parents_gpu(parent: torch.Tensor, block_m: int, max_ancestors: int, width: int, *,
+                                   check: bool = True, want_bool_mask: bool = False, want_lineage: bool = False,
+                                   status=None):
+    """``parent [N]`` int64 on the GPU -> the kernel inputs of ``create_fst_attention_kernel_inputs`` in ONE launch
+    (``fsta_precompute_from_parents``): what ``lineage_from_parents_gpu(parent, width)`` followed by
+    ``create_fst_attention_kernel_inputs(lineage, level, block_m, max_ancestors)`` returns, bit for bit, without the
+    lineage travelling through memory.  ``width``: columns of the lineage rows, at least the tree's depth + 1.
+    Returns ``(ancestor_idx, ancestor_mask or PackedTreeMask, leaf_idx)`` (``want_bool_mask`` as there), followed by
+    ``(lineage, level_lookup)`` with ``want_lineage`` (the lineage with the nodes' own ids entered, as the reference's
+    function leaves it) and by the device status word with ``check=False``.  Trees whose tables do not fit one
+    workgroup's LDS (about 16000 nodes) raise ``libfsta``'s unsupported error: use the two calls."""
+    if not parent.is_cuda or parent.dtype != torch.int64 or parent.dim() != 1:
+        raise ValueError("parent must be a 1-D int64 tensor on the GPU")
+    lib = _lib.load()
+    parent = parent.contiguous()
+    dev = parent.device
+    n, block_m, max_ancestors, width = parent.shape[0], int(block_m), int(max_ancestors), int(width)
+    nb = -(-n // block_m)
+    a_idx = torch.empty((nb, max_ancestors), dtype=torch.int64, device=dev)
+    l_idx = torch.empty((nb, block_m), dtype=torch.int64, device=dev)
+    a_mask = torch.empty((nb, block_m, max_ancestors), dtype=torch.bool, device=dev) if want_bool_mask else None
+    bits = torch.empty((nb, lib.fsta_mask_words(max_ancestors), block_m), dtype=torch.int32, device=dev)
+    count = torch.empty((nb,), dtype=torch.int32, device=dev)
+    plan_bytes = lib.fsta_block_plan_bytes(nb, block_m, max_ancestors)
+    plan = torch.empty((plan_bytes // 4,), dtype=torch.int32, device=dev) if plan_bytes else None
+    lineage = torch.empty((n, width), dtype=torch.int64, device=dev) if want_lineage else None
+    level = torch.empty((n,), dtype=torch.int64, device=dev) if want_lineage else None
+    if status is None:
+        status = torch.zeros((1,), dtype=torch.int32, device=dev)
+    ptr = lambda t: t.data_ptr() if t is not None else None
+    with _on_device(dev):
+        _lib.check(lib.fsta_precompute_from_parents(parent.data_ptr(), n, width, block_m, max_ancestors, 1, ptr(lineage),
+                                                    ptr(level), a_idx.data_ptr(), ptr(a_mask), l_idx.data_ptr(),
+                                                    bits.data_ptr(), count.data_ptr(), ptr(plan), status.data_ptr(),
+                                                    _stream_ptr(dev)))
+    if check:
+        st = int(status.item())
+        if st & _lib.PRE_BAD_LEVEL:
+            raise ValueError(f"tree is deeper than width={width}")
+        if st & _lib.PRE_BAD_NODE_ID:
+            raise ValueError("parent[i] must lie in [-1, i)")
+        _raise_for_status(st, max_ancestors)
+    packed = PackedTreeMask(bits, count, block_m, max_ancestors, plan)
+    if want_bool_mask:
+        key = _cache_key(a_idx, a_mask, l_idx)
+        if key is not None:
+            remember_packed(a_mask, key, packed)
+    out = (a_idx, a_mask if want_bool_mask else packed, l_idx)
+    if want_lineage:
+        out += (lineage, level)
+    return out if check else out + (status,)
+
+
 def lineage_from_parents_gpu(parent: torch.Tensor, width: Optional[int] = None, check: bool = True, status=None):
     """``parent [N]`` int64 on the GPU -> ``(lineage [N, width], level_lookup [N])`` on the GPU.
 

@@ -257,6 +257,30 @@ int fsta_lineage_from_parents(const int64_t* parent, int64_t n_nodes, int64_t wi
                               void* stream);
 
 /*
+ * fsta_lineage_from_parents and fsta_precompute in one launch, for the trees of a
+ * decoding step that is rebuilt every step (README.md:15-16): every workgroup
+ * copies parent[n_nodes] into its LDS, builds the lineage rows of its own query
+ * block there (layout of utils.py:66-75, `width` columns) and goes on as
+ * fsta_precompute does (utils.py:104-129), without the lineage ever travelling
+ * through memory.  Outputs and status bits are those of fsta_precompute on the
+ * lineage of fsta_lineage_from_parents, bit for bit; lineage [n_nodes, width] and
+ * level_lookup [n_nodes] are optional outputs here (NULL: not written), lineage
+ * with each node's id in its own level column when insert_self != 0 (what
+ * fsta_precompute leaves in the caller's tensor).  A tree deeper than width - 1
+ * sets FSTA_PRE_BAD_LEVEL, a parent entry outside [-1, i) FSTA_PRE_BAD_NODE_ID
+ * (such a node counts as a root).  Everything lives in one workgroup's LDS:
+ * 4 * (n_nodes + block_m * width) bytes beside fsta_precompute's tables, 160 KB in
+ * all -- about 16000 nodes at width 64, block_m 128; larger problems are refused
+ * with FSTA_EUNSUPPORTED (use the two calls).  No counterpart in the reference.
+ * Alignment as fsta_precompute; parent 8 bytes.
+ */
+int fsta_precompute_from_parents(const int64_t* parent, int64_t n_nodes, int64_t width, int32_t block_m,
+                                 int32_t max_ancestors, int32_t insert_self, int64_t* lineage,
+                                 int64_t* level_lookup, int64_t* ancestor_idx, uint8_t* ancestor_mask,
+                                 int64_t* leaf_idx, uint32_t* mask_bits, int32_t* anc_count,
+                                 uint32_t* block_plan, uint32_t* status, void* stream);
+
+/*
  * Depth-first (pre-order) renumbering of a forest, the node order the reference
  * names as its open item (README.md:19-20: blocks of consecutive ids then share
  * lineage and their ancestor lists shrink).  parent[n_nodes] int64 as above ->

@@ -4,7 +4,8 @@ import pytest
 import torch
 
 from conftest import golden_cases
-from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, lineage_from_parents_gpu,
+from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, kernel_inputs_from_parents_gpu,
+                              lineage_from_parents_gpu,
                               medusa_parents_gpu, pack_tree_mask, renumber_parents_gpu, trees)
 from fstattention_amd.attention import recall_packed
 from oracle import tree_precompute as tp
@@ -333,3 +334,35 @@ def test_device_only_pipeline_from_probabilities_to_kernel_inputs():
     lin, lvl = trees.lineage_from_parents(host_new, min_width=5)
     want = tp.block_inputs(lin.numpy().copy(), lvl.numpy(), 64, 64)
     _check(got, want)
+
+
+def test_kernel_inputs_from_parents_in_one_launch():
+    """``fsta_precompute_from_parents`` against the two-launch chain on the benchmark trees that fit one workgroup's
+    LDS (bit for bit, packed inputs and block plan included), its status bits, and its refusal of a tree too large."""
+    from fstattention_amd import _lib
+    for index in (2, 3, 4, 5):
+        cfg = trees.config(index)
+        parent = torch.from_numpy(cfg.parent).cuda()
+        max_anc = trees.required_max_ancestors(cfg.parent, cfg.block_m, 16)
+        lineage, level = lineage_from_parents_gpu(parent)
+        want_idx, want_packed, want_leaf = create_fst_attention_kernel_inputs(lineage, level, cfg.block_m, max_anc,
+                                                                              want_bool_mask=False)
+        a_idx, packed, l_idx, lin, lvl = kernel_inputs_from_parents_gpu(parent, cfg.block_m, max_anc, lineage.shape[1],
+                                                                        want_lineage=True)
+        assert torch.equal(a_idx, want_idx) and torch.equal(l_idx, want_leaf), cfg.name
+        assert torch.equal(packed.mask_bits, want_packed.mask_bits) and torch.equal(packed.anc_count, want_packed.anc_count)
+        assert torch.equal(packed.plan, want_packed.plan), cfg.name
+        assert torch.equal(lin, lineage) and torch.equal(lvl, level), cfg.name      # (lineage carries the self entries by now)
+    # too shallow rows, a malformed parent entry, too many ancestors: flagged, no fault
+    chain = torch.arange(-1, 99, dtype=torch.int64, device="cuda")
+    with pytest.raises(ValueError, match="deeper"):
+        kernel_inputs_from_parents_gpu(chain, 32, 128, 50)
+    bad = torch.from_numpy(trees.random_recursive_parents(300, 5, 16)).cuda()
+    bad[17] = 200
+    with pytest.raises(ValueError, match="parent"):
+        kernel_inputs_from_parents_gpu(bad, 64, 64, 64)
+    with pytest.raises(RuntimeError, match="max_ancestors"):
+        kernel_inputs_from_parents_gpu(chain, 32, 16, 128)
+    big = torch.from_numpy(trees.random_recursive_parents(60000, 6, 64)).cuda()
+    with pytest.raises(_lib.FstaError, match="LDS"):
+        kernel_inputs_from_parents_gpu(big, 128, 64, 64)

@@ -7,8 +7,10 @@ import numpy as np
 import pytest
 import torch
 
-from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, fst_attention,
+from fstattention_amd import (create_fst_attention_kernel_inputs, dfs_order_gpu, fst_attention, kernel_inputs_from_parents_gpu,
                               lineage_from_parents_gpu, pack_tree_mask, renumber_parents_gpu, shift_for_prefix, trees)
+from fstattention_amd import _lib
+from fstattention_amd.attention import recall_packed
 from helpers import TOL, dense_oracle, expected_plan, rand_qkv
 from oracle import tree_precompute as tp
 
@@ -73,7 +75,26 @@ def test_integer_front_end_sweep_is_bit_exact():
         for g_, w_ in zip(got, want):
             np.testing.assert_array_equal(g_.cpu().numpy(), w_, err_msg=what)
         np.testing.assert_array_equal(lin_dev.cpu().numpy(), lin_host, err_msg=what)     # utils.py:124-125
+        # the same from the parent array in one launch (lineage rows built in LDS)
         packed = pack_tree_mask(got[0], got[1], got[2])
+        fits = 4 * (2 * ((n + 31) // 32) + (max_anc + 31) // 32 * m + m + 4 + m * lineage.shape[1] + n) <= 160 * 1024
+        if fits:
+            fa, fm, fl, flin, flvl = kernel_inputs_from_parents_gpu(pt, m, max_anc, lineage.shape[1], want_bool_mask=True,
+                                                                    want_lineage=True)
+            for g_, w_ in zip((fa, fm, fl), want):
+                np.testing.assert_array_equal(g_.cpu().numpy(), w_, err_msg="one launch, " + what)
+            np.testing.assert_array_equal(flin.cpu().numpy(), lin_host, err_msg="one launch, " + what)
+            np.testing.assert_array_equal(flvl.cpu().numpy(), level.numpy(), err_msg="one launch, " + what)
+            fused_packed = recall_packed(fm)[1]
+            np.testing.assert_array_equal(fused_packed.mask_bits.cpu().numpy(), packed.mask_bits.cpu().numpy(), err_msg=what)
+            np.testing.assert_array_equal(fused_packed.anc_count.cpu().numpy(), packed.anc_count.cpu().numpy(), err_msg=what)
+            if m >= 32:
+                plan_want, care = expected_plan(*want)
+                plan_fused = fused_packed.plan.cpu().numpy().view(np.uint32).reshape(plan_want.shape[0], -1)
+                np.testing.assert_array_equal(plan_fused[care], plan_want[care], err_msg="one launch, " + what)
+        else:       # tables beyond one workgroup's LDS: refused on the host
+            with pytest.raises(_lib.FstaError, match="LDS"):
+                kernel_inputs_from_parents_gpu(pt, m, max_anc, lineage.shape[1])
         if m >= 32:
             plan_want, care = expected_plan(*want)
             plan_got = packed.plan.cpu().numpy().view(np.uint32).reshape(plan_want.shape[0], -1)
