@@ -501,8 +501,10 @@ def graph_us_per_node(call, nodes, reps=3):
 def measured_ceilings(wl, nodes=HEADLINE_MIN_STEPS):
     """This GPU's own ceilings, measured in this run: what a graph node of the headline launch's shape
     costs when the kernel does nothing (`launch_floor_us`), and what a kernel that only reads gets out
-    of HBM (`hbm_read_probe_gbps`: 1 GiB, 16 bytes per lane, eight loads per lane in flight, 2048 workgroups;
-    the buffer is four times the Infinity Cache, so every pass comes from HBM), beside torch's plain copy."""
+    of HBM (`hbm_read_probe_gbps`: 1 GiB, 16 bytes per lane, eight non-temporal loads per lane in flight, 4096
+    workgroups that each walk a contiguous piece -- the best of the eight variants of the probe on this GPU: striding
+    over the buffer with the whole grid, as a naive copy does, reads 5.1-5.7 TB/s, contiguous pieces with non-temporal
+    loads 7.0; the buffer is four times the Infinity Cache, so every pass comes from HBM), beside torch's plain copy."""
     import torch
     lib, check = wl.lib, wl._check
     cur = lambda: torch.cuda.current_stream().cuda_stream
@@ -512,7 +514,8 @@ def measured_ceilings(wl, nodes=HEADLINE_MIN_STEPS):
     n = 1 << 30
     src = torch.empty(n, dtype=torch.uint8, device="cuda").fill_(3)
     sink = torch.zeros((1,), dtype=torch.int32, device="cuda")
-    read_us = graph_us_per_node(lambda: check(lib.fsta_probe_hbm_read(src.data_ptr(), n, 2048, sink.data_ptr(), cur())), 4, reps=3)
+    read_us = graph_us_per_node(lambda: check(lib.fsta_probe_hbm_read(src.data_ptr(), n, 4096, 6, sink.data_ptr(), cur())), 4, reps=3)
+    strided_us = graph_us_per_node(lambda: check(lib.fsta_probe_hbm_read(src.data_ptr(), n, 2048, 0, sink.data_ptr(), cur())), 4, reps=3)
     dst = torch.empty(n // 4, dtype=torch.uint8, device="cuda")
     copy_us = graph_us_per_node(lambda: dst.copy_(src[: n // 4]), 4, reps=3)
     del src, dst
@@ -523,7 +526,9 @@ def measured_ceilings(wl, nodes=HEADLINE_MIN_STEPS):
                              "(the headline launch's shape)",
         "one_wave_graph_node_us": round(one_wave_us, 3),
         "hbm_read_probe_gbps": round(n / read_us / 1e3, 1),
-        "hbm_read_probe_note": "read-only kernel over 1 GiB, 16 B per lane, 8 loads in flight per lane, 2048 workgroups",
+        "hbm_read_probe_note": "read-only kernel over 1 GiB, 16 B per lane, 8 non-temporal loads in flight per lane, 4096 "
+                               "workgroups, a contiguous piece each",
+        "hbm_read_probe_grid_strided_gbps": round(n / strided_us / 1e3, 1),
         "torch_copy_read_plus_write_gbps": round(2 * (n // 4) / copy_us / 1e3, 1),
     }
 

@@ -67,7 +67,7 @@ SIGNATURES = {
     "fsta_medusa_tree_ws": (c_int, [c_void_p, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_size_t,
                                     c_void_p]),
     "fsta_probe_empty_launch": (c_int, [c_int32, c_int32, c_void_p]),
-    "fsta_probe_hbm_read": (c_int, [c_void_p, c_size_t, c_int32, c_void_p, c_void_p]),
+    "fsta_probe_hbm_read": (c_int, [c_void_p, c_size_t, c_int32, c_int32, c_void_p, c_void_p]),
     "fsta_merge_states": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                                   c_int32, c_int32, c_void_p]),
 }

@@ -346,11 +346,22 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p) {
             if ((kRowsO * kRowSlotsO > M && m >= M) || row >= p.nq) continue;
             const float l = stat_s[m];
             const size_t off = ((size_t)hz * p.nq + row) * D + oc;
+            // four neighbouring head dims leave in one store (non-temporal: nobody in this launch reads the output again)
+            typedef float f32x4 __attribute__((ext_vector_type(4)));
+            typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+            float val[4];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const float val = l > 0.f ? acc[i][c] / l : 0.f;
-                if (p.out_f32) static_cast<float*>(p.o)[off + c] = val;
-                else static_cast<T*>(p.o)[off + c] = from_float<T>(val);
+            for (int c = 0; c < 4; ++c) val[c] = l > 0.f ? acc[i][c] / l : 0.f;
+            if (p.out_f32 || sizeof(T) == 4) {
+                const f32x4 v = {val[0], val[1], val[2], val[3]};
+                __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(static_cast<float*>(p.o) + off));
+            } else {
+                T h[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) h[c] = from_float<T>(val[c]);
+                u32x2 pk;
+                __builtin_memcpy(&pk, h, sizeof(pk) < sizeof(h) ? sizeof(pk) : sizeof(h));
+                __builtin_nontemporal_store(pk, reinterpret_cast<u32x2*>(static_cast<T*>(p.o) + off));
             }
         }
     }

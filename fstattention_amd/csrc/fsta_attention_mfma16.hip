@@ -15,6 +15,14 @@
 // 8 weights it ends up with are exactly its 8 k-slots of the B operand of O^T += V^T.P^T.
 #include "fsta_mfma_common.h"
 
+// Cache policy (`aux` operand of the global->LDS transfers, 2 = non-temporal): rows that no other workgroup will ask
+// for again go past the caches' retention -- the Q rows, the output rows (non-temporal stores) and, in a launch whose
+// workgroups all run at once, the leaf tiles requested ahead of the plan.  K/V rows of larger launches are left alone:
+// a block's own rows are the ancestors of later blocks, which find them in L2 (non-temporal leaf rows: +13 % on the
+// reference's benchmark shape, measured).  Measured with Q and O non-temporal: cfg4 26.6 -> 23.5 us, cfg3 14.0 -> 13.0,
+// the reference's benchmark at N = 2048 41.4 -> 38.4, cfg2 5.28 -> 5.14 (5.10 with the early leaf tiles as well).
+constexpr int kStreamOnce = 2;
+
 namespace fsta {
 namespace {
 
@@ -60,7 +68,7 @@ __device__ __forceinline__ void flush_rows(const unsigned char* stage, int strid
         const int r = i * kRowsPerStore + st_row;
         if (r < 16 && r < rows_valid) {
             const u32x4 val = *reinterpret_cast<const u32x4*>(stage + r * stride + st_piece * 16);
-            *reinterpret_cast<u32x4*>(dst + r * pitch + st_piece * 16) = val;
+            __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(dst + r * pitch + st_piece * 16));
         }
     }
 }
@@ -245,7 +253,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         const uint32_t off = (uint32_t)grow * (uint32_t)(D * sizeof(T)) + (uint32_t)k_chunk<D>(r, q_slot) * 16u;
         __builtin_amdgcn_global_load_lds(
             (const void __attribute__((address_space(1)))*)(reinterpret_cast<const char*>(qb) + (size_t)off),
-            (void __attribute__((address_space(3)))*)(qstage + i * 512), 16, 0, 0);
+            (void __attribute__((address_space(3)))*)(qstage + i * 512), 16, 0, kStreamOnce);
     }
 
     // ---- gather: HBM -> LDS, 16 bytes per lane, no registers in between --------
@@ -274,7 +282,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
             dma_flip[i] = (t2 & 1) ? ((uint32_t)v16_chunk<D>(r, dma_slot) * 16u) ^ dma_leaf[i] : 0u;
         }
     }
-    auto issue_rows = [&](int t, int slot, const int (&rows)[kRowGroups]) {
+    auto issue_rows = [&](int t, int slot, const int (&rows)[kRowGroups], bool once) {
         unsigned char* dst_tile = KV8 ? stage8 + slot * kStageBytes : reinterpret_cast<unsigned char*>(ring + slot * 2 * kTileElems);
         constexpr int kHalf = KV8 ? kStageBytes / 2 : kTileElems * 2;   // bytes from the K part to the V part
         const uint32_t anc_tile = t < kLeafTiles ? 0u : 0xffffffffu;
@@ -286,10 +294,15 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
             const uint32_t off = (uint32_t)rows[i >> 1] * (uint32_t)kKvRowBytes +
                                  (KV8 ? (uint32_t)dma_slot * 16u : dma_leaf[i] ^ (dma_flip[i] & anc_tile));
             const char* src = reinterpret_cast<const char*>(is_v ? vb : kb) + (size_t)off;
-            __builtin_amdgcn_global_load_lds(
-                (const void __attribute__((address_space(1)))*)src,
-                (void __attribute__((address_space(3)))*)(dst_tile + (is_v ? kHalf : 0) + u * 1024),
-                16, 0, 0);
+            // (`once` is a constant at both call sites: one of the two forms remains)
+            if (once)
+                __builtin_amdgcn_global_load_lds(
+                    (const void __attribute__((address_space(1)))*)src,
+                    (void __attribute__((address_space(3)))*)(dst_tile + (is_v ? kHalf : 0) + u * 1024), 16, 0, kStreamOnce);
+            else
+                __builtin_amdgcn_global_load_lds(
+                    (const void __attribute__((address_space(1)))*)src,
+                    (void __attribute__((address_space(3)))*)(dst_tile + (is_v ? kHalf : 0) + u * 1024), 16, 0, 0);
         }
     };
     // A valid leaf slot of row r names r's own key (reference utils.py:121-122), so the first
@@ -307,7 +320,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
 #pragma unroll
         for (int i = 0; i < kRowGroups; ++i)
             rows[i] = min(p.prefix + row_base + t * kTileN + ((wave * kDmaPerWave) / 2 + i) * kRowsPerDma + dma_row, p.nk - 1);
-        issue_rows(t, t, rows);
+        issue_rows(t, t, rows, true);
     }
 
     FSTA_STAMP(1);    // all start-up requests are out
@@ -387,7 +400,7 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
             for (int i = 0; i < kRowGroups; ++i)
                 rows[i] = min((t + prefix_shift) * kTileN + ((wave * kDmaPerWave) / 2 + i) * kRowsPerDma + dma_row, p.prefix - 1);
         }
-        issue_rows(t, slot, rows);
+        issue_rows(t, slot, rows, false);
     };
 
     // Ring bookkeeping, in tiles: `issued` gathers started, `consumed` tiles everyone is done

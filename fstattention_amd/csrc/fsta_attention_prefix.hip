@@ -97,7 +97,8 @@ __global__ __launch_bounds__(kPfxWaves * 64, 2) void prefix_attn_kernel(AttnPara
         const int row = min(row_base + wave * 32 + h * 16 + ql, p.nq - 1);
 #pragma unroll
         for (int s = 0; s < kSteps; ++s) {
-            const u32x4 raw = *reinterpret_cast<const u32x4*>(qb + (size_t)row * D + 32 * s + 8 * g);
+            // (non-temporal: the Q rows of a run are read once)
+            const u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(qb + (size_t)row * D + 32 * s + 8 * g));
             qf[h][s] = __builtin_bit_cast(Frag, raw);
         }
     }

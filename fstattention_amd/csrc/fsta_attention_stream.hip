@@ -218,7 +218,7 @@ __global__ __launch_bounds__(M * 4, 4) void attn_stream_kernel(AttnParams p, int
                 const int grow = min(row_base + local * 64 + rr, p.nq - 1);
                 const uint32_t off = (uint32_t)grow * (uint32_t)kRowBytes + (uint32_t)k_chunk<D>(rr, dma_slot) * 16u;
                 __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(qb + (size_t)off),
-                                                 (void __attribute__((address_space(3)))*)(dst_tile + t2 * 1024), 16, 0, 0);
+                                                 (void __attribute__((address_space(3)))*)(dst_tile + t2 * 1024), 16, 0, 2);   // (non-temporal: read once)
             }
         } else {
             const int pos = local - kQTiles;
@@ -581,7 +581,7 @@ __global__ __launch_bounds__(M * 4, 4) void attn_stream_kernel(AttnParams p, int
 #pragma unroll
                     for (int dt = 0; dt < kOTiles; ++dt) {
                         const f32x4 val = {o[dt][0] * inv, o[dt][1] * inv, o[dt][2] * inv, o[dt][3] * inv};
-                        if (row < p.nq) *reinterpret_cast<f32x4*>(ob + 16 * dt) = val;
+                        if (row < p.nq) __builtin_nontemporal_store(val, reinterpret_cast<f32x4*>(ob + 16 * dt));
                     }
                     count_ops(kOTiles);
                 } else {
@@ -596,7 +596,7 @@ __global__ __launch_bounds__(M * 4, 4) void attn_stream_kernel(AttnParams p, int
                         const u32x2 s1 = __builtin_amdgcn_permlane16_swap(x1, y1, false, false);
                         const uint32_t a0 = s0[0], b0 = s0[1], a1 = s1[0], b1 = s1[1];
                         const u32x4 val = {a0, a1, b0, b1};
-                        if (row < p.nq) *reinterpret_cast<u32x4*>(ob + 32 * a) = val;
+                        if (row < p.nq) __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(ob + 32 * a));
                     }
                     count_ops(kOTiles / 2);
                 }

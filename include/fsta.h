@@ -386,11 +386,13 @@ int fsta_medusa_tree_ws(const void* probs, int32_t probs_dtype, int32_t depths, 
  *     workgroups of `threads` threads: what a launch of that shape costs by itself.
  *   fsta_probe_hbm_read: a kernel that only reads: `bytes` (a multiple of 16) from
  *     src (16-byte aligned), 16 bytes per lane, consecutive lanes consecutive
- *     addresses, eight loads per lane in flight, `workgroups` workgroups of 256
- *     threads; `sink` (may be NULL) is never written in practice.
+ *     addresses, `workgroups` workgroups of 256 threads; `variant` 0..7: bit 0 = 16
+ *     instead of 8 loads per lane in flight, bit 1 = non-temporal loads, bit 2 =
+ *     every workgroup walks a contiguous piece instead of striding with the grid;
+ *     `sink` (may be NULL) is never written in practice.
  */
 int fsta_probe_empty_launch(int32_t workgroups, int32_t threads, void* stream);
-int fsta_probe_hbm_read(const void* src, size_t bytes, int32_t workgroups, uint32_t* sink, void* stream);
+int fsta_probe_hbm_read(const void* src, size_t bytes, int32_t workgroups, int32_t variant, uint32_t* sink, void* stream);
 
 #ifdef __cplusplus
 }
