@@ -154,7 +154,8 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     // A workgroup takes M consecutive rows: a whole block of the caller's, or (sub_shift = 1, small
     // grids) one half of a block of 2M rows, so that twice as many CUs share the launch.  The
     // half-block reads the block's ancestor list and its own rows of the mask and leaf list.
-    const int linear_grid = sub_shift >> 8;
+    const int linear_grid = (sub_shift >> 8) & 1;
+    const int late_first = (sub_shift >> 9) & 1;
     sub_shift &= 0xff;
     const int xcd = blockIdx.x % kXcds;
     int ksp = 0, hz, part;
@@ -171,6 +172,13 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         if constexpr (RUNS) ksp = blockIdx.x / kXcds;
         hz = blockIdx.z * kXcds + xcd;
         part = blockIdx.y;
+        if (late_first) {
+            // (8 XCDs, slices per XCD, blocks): the late blocks of every slice, which have the longest
+            // ancestor lists, are dispatched first, so that the two workgroups that come to share a CU in a
+            // launch of more than one and at most two per CU are one of the long and one of the short half.
+            hz = blockIdx.y * kXcds + xcd;
+            part = gridDim.z - 1 - blockIdx.z;
+        }
     }
     const bool tree = !RUNS || ksp == 0;
     const int j = part >> sub_shift;                                        // block of the caller's lists
@@ -920,9 +928,12 @@ int launch_ks(const AttnParams& p, int sub_shift, hipStream_t stream) {
     const unsigned grid = (unsigned)(kXcds * slices_per_xcd * (p.nb << sub_shift) * p.key_splits);   // workgroups
     // (8 XCDs x key runs, blocks, slices per XCD) where the y and z extents allow it, else one axis
     const bool linear_grid = (p.nb << sub_shift) > 65535 || slices_per_xcd > 65535;
-    const dim3 grid3 = linear_grid ? dim3(grid)
-                                   : dim3((unsigned)(kXcds * p.key_splits), (unsigned)(p.nb << sub_shift), (unsigned)slices_per_xcd);
-    const int shift_arg = sub_shift | (linear_grid ? 0x100 : 0);
+    // More than one and at most two workgroups per CU: late blocks first (see the kernel's mapping).
+    const bool late_first = !linear_grid && !p.part_o && p.key_splits == 1 && grid > (unsigned)kCus && grid <= 2u * kCus;
+    const dim3 grid3 = linear_grid  ? dim3(grid)
+                       : late_first ? dim3((unsigned)kXcds, (unsigned)slices_per_xcd, (unsigned)(p.nb << sub_shift))
+                                    : dim3((unsigned)(kXcds * p.key_splits), (unsigned)(p.nb << sub_shift), (unsigned)slices_per_xcd);
+    const int shift_arg = sub_shift | (linear_grid ? 0x100 : 0) | (late_first ? 0x200 : 0);
     // a launch whose workgroups all run at once: leaf tiles requested early, Q in an area of its own
     constexpr size_t kQBytes = (size_t)kWaves * 16 * D * 2;
     const int early = grid <= kCus && !p.part_o && lds + kQBytes <= 160 * 1024 ? 1 : 0;
