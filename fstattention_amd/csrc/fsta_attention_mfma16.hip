@@ -14,6 +14,7 @@
 // query, so a lane owns keys 4g .. 4g+3 of each 16-key half of a tile for ONE query, and the
 // 8 weights it ends up with are exactly its 8 k-slots of the B operand of O^T += V^T.P^T.
 #include "fsta_mfma_common.h"
+#include <type_traits>
 
 // Cache policy (`aux` operand of the global->LDS transfers, 2 = non-temporal): rows that no other workgroup will ask
 // for again go past the caches' retention -- the Q rows, the output rows (non-temporal stores) and, in a launch whose
@@ -616,49 +617,35 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
     const uint32_t v_lane0 = (uint32_t)(tr_r0 * D + v16_chunk<D>(tr_r0, tr_col >> 3) * 8 + (tr_col & 7)) * 2;
     // this row's mask words, one per ancestor tile (bits of empty slots are clear in the plan)
     const uint32_t* my_mask = group_s + (row_in_block >> 5) * group_words + kTileN + (row_in_block & 31);
-    while (consumed < total_tiles) {
-#ifdef FSTA_TIMELINE
-        if (tl_tile < 5) { FSTA_STAMP(7 + tl_tile); }     // begin of ancestor / prefix step tl_tile
-        ++tl_tile;
-#endif
-        begin_step(kSplit);
-        const int t = consumed + (kDShare ? 0 : split);
-        const T* kt = tile_ptr(kDShare ? 0 : split);
-        const T* vt = kt + kTileElems;
-        end_step(kSplit);
-        uint32_t word = 0u;
-        if (t < listed_tiles) {
-            word = my_mask[(t - kLeafTiles) * kTileN];
-        } else if (t < total_tiles) {
-            const int left = p.prefix - (t + prefix_shift) * kTileN;
-            word = left >= 32 ? 0xffffffffu : ((1u << left) - 1u);
-        }
-        if (kSplit > 1 && t >= total_tiles) continue;   // this share has no tile in the last step
-        // A tile none of this wave's 16 queries attends to (10-30 % of the ancestor tiles of deep
-        // trees) is skipped where a workgroup walks long lists; in the short chains of the
-        // head-dimension pairing the branch costs more than the rare skip saves.
-        if (!kDShare && __ballot(word != 0u) == 0ull) continue;
-
-        // S^T = K_tile . Q^T, two halves of 16 keys
-        typedef const u32x4 __attribute__((address_space(3))) * lds_u32x4;
-        const uint32_t k_addr0 = lds_addr(kt) + k_lane0;
-        f32x4 s[2];
+    // One step of NT tiles (32 keys each) for this wave: S^T, mask, weights, O^T.  NT = 2 (the waves that share
+    // the head dimension: short lists, every tile in LDS before the first step) treats two tiles as one of 64
+    // keys: one pass through the weights, one check of the running maximum, one chain MFMA -> vector ALU -> MFMA
+    // instead of two, which is what a lone wave on its SIMD waits for.
+    typedef const u32x4 __attribute__((address_space(3))) * lds_u32x4;
+    constexpr int kHalf = kOTiles / 2;
+    auto step_tiles = [&](auto nt_tag, const T* const (&kts)[2], const uint32_t (&words)[2]) {
+        constexpr int NT = decltype(nt_tag)::value;
+        // S^T = K_tile . Q^T, two halves of 16 keys per tile
+        f32x4 s[2 * NT];
 #pragma unroll
-        for (int sub = 0; sub < 2; ++sub) {
-            s[sub] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int tl = 0; tl < NT; ++tl) {
+            const uint32_t k_addr0 = lds_addr(kts[tl]) + k_lane0;
 #pragma unroll
-            for (int ks = 0; ks < kSteps; ++ks) {
-                const u32x4 raw = *(lds_u32x4)(uintptr_t)((k_addr0 ^ (uint32_t)(ks << 6)) + sub * kHalfTileBytes);
-                s[sub] = mfma16(__builtin_bit_cast(Frag, raw), qf[ks], s[sub]);
+            for (int sub = 0; sub < 2; ++sub) {
+                s[2 * tl + sub] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < kSteps; ++ks) {
+                    const u32x4 raw = *(lds_u32x4)(uintptr_t)((k_addr0 ^ (uint32_t)(ks << 6)) + sub * kHalfTileBytes);
+                    s[2 * tl + sub] = mfma16(__builtin_bit_cast(Frag, raw), qf[ks], s[2 * tl + sub]);
+                }
             }
         }
         // V fragments (A operand of O^T += V^T.P^T: rows are head dims) through the transposing
         // read: k-slots 8g .. 8g+3 are keys 4g .. 4g+3, k-slots 8g+4 .. 8g+7 keys 16+4g .. 16+4g+3.
         // Half of the head-dim tiles are requested now (LDS latency hides behind the softmax),
         // the other half behind the first MFMAs.
-        constexpr int kHalf = kOTiles / 2;
-        const uint32_t v_addr0 = lds_addr(vt) + v_lane0;
-        auto read_v = [&](VPair (&f)[kHalf], int first_dt) {
+        auto read_v = [&](VPair (&f)[kHalf], const T* vt, int first_dt) {
+            const uint32_t v_addr0 = lds_addr(vt) + v_lane0;
 #pragma unroll
             for (int i = 0; i < kHalf; ++i) {
                 const uint32_t addr = v_addr0 ^ (uint32_t)((first_dt + i) << 5);
@@ -672,38 +659,44 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
             for (int i = 0; i < kHalf; ++i) { lds_tie(f[i].a); lds_tie(f[i].b); }
         };
         VPair v0[kHalf], v1[kHalf];
-        read_v(v0, dt0);
+        read_v(v0, kts[0] + kTileElems, dt0);
         // mask + online softmax; register j of half `sub` is key 16*sub + 4g + j.  The scale rides
         // in the FMA under the exp2.
-        const uint32_t wsh = word >> (4 * g);
-        float sv[8];
+        float sv[8 * NT];
+        uint32_t own_bits = 0u;   // mask bits of the keys this lane holds
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
-            // bit -> all-ones / all-zeros (v_bfe_i32), then a bitwise select against -inf (v_bfi_b32)
-            const uint32_t keep = (uint32_t)__builtin_amdgcn_sbfe((int)wsh, 16 * (r / 4) + (r % 4), 1);
-            const float score = s[r / 4][r % 4];   // (a copy: bit_cast straight from a vector element reads element 0)
-            const uint32_t bits = __builtin_bit_cast(uint32_t, score);
-            sv[r] = __builtin_bit_cast(float, (bits & keep) | (0xff800000u & ~keep));
+        for (int tl = 0; tl < NT; ++tl) {
+            const uint32_t wsh = words[tl] >> (4 * g);
+            own_bits |= wsh & 0x000f000fu;
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                // bit -> all-ones / all-zeros (v_bfe_i32), then a bitwise select against -inf (v_bfi_b32)
+                const uint32_t keep = (uint32_t)__builtin_amdgcn_sbfe((int)wsh, 16 * (r / 4) + (r % 4), 1);
+                const float score = s[2 * tl + r / 4][r % 4];   // (a copy: bit_cast straight from a vector element reads element 0)
+                const uint32_t bits = __builtin_bit_cast(uint32_t, score);
+                sv[8 * tl + r] = __builtin_bit_cast(float, (bits & keep) | (0xff800000u & ~keep));
+            }
         }
         // The weights are first taken against the running maximum as it stands: no row maximum,
         // no cross-lane exchange.  That is exact as long as no weight gets large (a power-of-two
         // factor on a row's weights cancels in O / l); the sum of the lane's weights is the check.
         // A row without a maximum so far, or a sum above the limit (or not a number), sends the
         // wave through the full update below: row maximum, raise, rescale, weights again.
-        float pw[8];
+        float pw[8 * NT];
         float rowsum = 0.f;
         {
             const float neg_m = m_i == -INFINITY ? 0.f : -m_i;
 #pragma unroll
-            for (int r = 0; r < 8; ++r) {
+            for (int r = 0; r < 8 * NT; ++r) {
                 pw[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[r], sc, neg_m));
                 rowsum += pw[r];
             }
         }
-        const bool redo = !(rowsum <= kTrustedSum) || (m_i == -INFINITY && (wsh & 0x000f000fu) != 0u);
+        const bool redo = !(rowsum <= kTrustedSum) || (m_i == -INFINITY && own_bits != 0u);
         if (__ballot(redo) != 0ull) {
-            float mx_raw = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
-                                 fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+            float mx_raw = sv[0];
+#pragma unroll
+            for (int r = 1; r < 8 * NT; ++r) mx_raw = fmaxf(mx_raw, sv[r]);
             mx_raw = max_quarters(mx_raw);
             const float mx = mx_raw * sc;   // the scale is positive here
             // raise only rows that would otherwise keep a weight above 2^kRescaleSlack
@@ -718,39 +711,87 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
             const float neg_m = m_i == -INFINITY ? 0.f : -m_i;
             rowsum = 0.f;
 #pragma unroll
-            for (int r = 0; r < 8; ++r) {
+            for (int r = 0; r < 8 * NT; ++r) {
                 pw[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[r], sc, neg_m));
                 rowsum += pw[r];
             }
         }
         l_i += rowsum;
-        // P^T fragment: the 8 weights are this lane's 8 k-slots
-        u32x4 hi4, lo4;
+        // P^T fragments: the 8 weights of a tile are this lane's 8 k-slots
+        Frag ph[NT], pl[NT];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const float a = pw[2 * e], b = pw[2 * e + 1];
-            const uint32_t hi = MM::pack(a, b);
-            hi4[e] = hi;
-            if (SPLIT) lo4[e] = MM::pack(a - MM::low(hi), b - MM::high(hi));
+        for (int tl = 0; tl < NT; ++tl) {
+            u32x4 hi4, lo4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float a = pw[8 * tl + 2 * e], b = pw[8 * tl + 2 * e + 1];
+                const uint32_t hi = MM::pack(a, b);
+                hi4[e] = hi;
+                if (SPLIT) lo4[e] = MM::pack(a - MM::low(hi), b - MM::high(hi));
+            }
+            ph[tl] = __builtin_bit_cast(Frag, hi4);
+            if (SPLIT) pl[tl] = __builtin_bit_cast(Frag, lo4);
         }
-        const Frag ph = __builtin_bit_cast(Frag, hi4);
-        Frag pl;
-        if (SPLIT) pl = __builtin_bit_cast(Frag, lo4);
         // O^T += V_tile^T . P^T
-        tie_v(v0);
-        read_v(v1, dt0 + kHalf);
 #pragma unroll
-        for (int i = 0; i < kHalf; ++i) o[i] = mfma16(__builtin_bit_cast(Frag, v0[i]), ph, o[i]);
-        if (SPLIT) {
+        for (int tl = 0; tl < NT; ++tl) {
+            tie_v(v0);
+            read_v(v1, kts[tl] + kTileElems, dt0 + kHalf);
 #pragma unroll
-            for (int i = 0; i < kHalf; ++i) o[i] = mfma16(__builtin_bit_cast(Frag, v0[i]), pl, o[i]);
+            for (int i = 0; i < kHalf; ++i) o[i] = mfma16(__builtin_bit_cast(Frag, v0[i]), ph[tl], o[i]);
+            if (SPLIT) {
+#pragma unroll
+                for (int i = 0; i < kHalf; ++i) o[i] = mfma16(__builtin_bit_cast(Frag, v0[i]), pl[tl], o[i]);
+            }
+            tie_v(v1);
+            if (tl + 1 < NT) read_v(v0, kts[tl + 1] + kTileElems, dt0);
+#pragma unroll
+            for (int i = 0; i < kHalf; ++i) o[kHalf + i] = mfma16(__builtin_bit_cast(Frag, v1[i]), ph[tl], o[kHalf + i]);
+            if (SPLIT) {
+#pragma unroll
+                for (int i = 0; i < kHalf; ++i) o[kHalf + i] = mfma16(__builtin_bit_cast(Frag, v1[i]), pl[tl], o[kHalf + i]);
+            }
         }
-        tie_v(v1);
-#pragma unroll
-        for (int i = 0; i < kHalf; ++i) o[kHalf + i] = mfma16(__builtin_bit_cast(Frag, v1[i]), ph, o[kHalf + i]);
-        if (SPLIT) {
-#pragma unroll
-            for (int i = 0; i < kHalf; ++i) o[kHalf + i] = mfma16(__builtin_bit_cast(Frag, v1[i]), pl, o[kHalf + i]);
+    };
+    while (consumed < total_tiles) {
+#ifdef FSTA_TIMELINE
+        if (tl_tile < 5) { FSTA_STAMP(7 + tl_tile); }     // begin of ancestor / prefix step tl_tile
+        ++tl_tile;
+#endif
+        if constexpr (kDShare) {
+            // (no prefix, no skipping: the launch code sends only short ancestor lists here)
+            const int n_here = total_tiles - consumed >= 2 ? 2 : 1;
+            begin_step(n_here);
+            const T* const kts[2] = {tile_ptr(0), tile_ptr(1)};
+            const int t = consumed;
+            end_step(n_here);
+            const uint32_t w0 = t < listed_tiles ? my_mask[(t - kLeafTiles) * kTileN] : 0u;
+            if (n_here == 2) {
+                const uint32_t w1 = t + 1 < listed_tiles ? my_mask[(t + 1 - kLeafTiles) * kTileN] : 0u;
+                const uint32_t words[2] = {w0, w1};
+                step_tiles(std::integral_constant<int, 2>{}, kts, words);
+            } else {
+                const uint32_t words[2] = {w0, 0u};
+                step_tiles(std::integral_constant<int, 1>{}, kts, words);
+            }
+        } else {
+            begin_step(kSplit);
+            const int t = consumed + split;
+            const T* const kts[2] = {tile_ptr(split), nullptr};
+            end_step(kSplit);
+            uint32_t word = 0u;
+            if (t < listed_tiles) {
+                word = my_mask[(t - kLeafTiles) * kTileN];
+            } else if (t < total_tiles) {
+                const int left = p.prefix - (t + prefix_shift) * kTileN;
+                word = left >= 32 ? 0xffffffffu : ((1u << left) - 1u);
+            }
+            if (kSplit > 1 && t >= total_tiles) continue;   // this share has no tile in the last step
+            // A tile none of this wave's 16 queries attends to (10-30 % of the ancestor tiles of deep
+            // trees) is skipped where a workgroup walks long lists.
+            if (__ballot(word != 0u) == 0ull) continue;
+            const uint32_t words[2] = {word, 0u};
+            step_tiles(std::integral_constant<int, 1>{}, kts, words);
         }
     }
 
