@@ -37,6 +37,7 @@ def main():
     ap.add_argument("--config", type=int, default=2)
     ap.add_argument("--warm", action="store_true", help="run the launch twice on the same buffers and time the second")
     ap.add_argument("--stream", action="store_true", help="the streaming kernel's cycle shares instead")
+    ap.add_argument("--slowest", type=int, default=0, help="also print the points of the N waves that end last")
     args = ap.parse_args()
     if not os.path.exists(TIMELINE_LIB_PATH):
         raise SystemExit(f"{TIMELINE_LIB_PATH} is missing: python -m fstattention_amd.build --timeline")
@@ -105,6 +106,12 @@ def main():
     start = (real[:, 0] - real[:, 0].min()) / 100.0
     end = (real[:, 1] - real[:, 0].min()) / 100.0
     print(f"waves start over {start.max():.2f} us (mean {start.mean():.2f}); the last one ends {end.max():.2f} us after the first started")
+    if args.slowest:
+        # the waves that end last set the launch's time: their own points, in us since their entry
+        print(f"the {args.slowest} waves that end last (entry in us after the first wave's, then us since entry at every point reached):")
+        for w in np.argsort(end)[::-1][:args.slowest]:
+            pts = " ".join(f"{i}:{rel[w, i] / 100.0:.2f}" for i in (1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 15, 13, 14) if ticks[w, i] != 0)
+            print(f"  entry {start[w]:.2f}  {pts}  exit {life_us[w]:.2f}")
 
 
 SEGMENTS = ["wait for the step's tile (vmcnt)", "workgroup barrier", "plan published, next tile requested (scalar bookkeeping)",
