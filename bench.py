@@ -345,20 +345,23 @@ def time_front_end(index, reps=20, stages=None):
             torch.cuda.synchronize()
         return round(ev0.elapsed_time(ev1) * 1e3 / reps, 2)
 
+    # the status word the stages of a step share: zeroed once per step by the caller, not by every stage
+    st = torch.zeros((1,), dtype=torch.int32, device=dev)
     calls = {
-        "dfs_order_us": lambda: dfs_order_gpu(parent, "light_first", check=False),
-        "lineage_from_parents_us": lambda: lineage_from_parents_gpu(parent, width=width, check=False),
+        "dfs_order_us": lambda: dfs_order_gpu(parent, "light_first", check=False, status=st),
+        "lineage_from_parents_us": lambda: lineage_from_parents_gpu(parent, width=width, check=False, status=st),
         "kernel_inputs_us": lambda: create_fst_attention_kernel_inputs(
-            lineage, level, cfg.block_m, max_anc, mutate_lineage=False, check=False, want_bool_mask=False),
+            lineage, level, cfg.block_m, max_anc, mutate_lineage=False, check=False, want_bool_mask=False, status=st),
         # the two stages above in one launch (lineage rows built in every workgroup's LDS)
-        "kernel_inputs_from_parents_us": lambda: kernel_inputs_from_parents_gpu(parent, cfg.block_m, max_anc, width, check=False),
+        "kernel_inputs_from_parents_us": lambda: kernel_inputs_from_parents_gpu(parent, cfg.block_m, max_anc, width, check=False,
+                                                                                status=st),
     }
     if index == 2:
         probs = torch.from_numpy(trees.medusa_probs()).to(dev)
-        calls["tree_from_probabilities_us"] = lambda: medusa_parents_gpu(probs, cfg.n_nodes)
+        calls["tree_from_probabilities_us"] = lambda: medusa_parents_gpu(probs, cfg.n_nodes, status=st)
         # five draft depths of 10 ranks: 111110 candidate paths, the multi-launch builder over a workspace
         probs5 = torch.from_numpy(trees.medusa_probs(5, 10)).to(dev)
-        calls["tree_from_probabilities_111110_paths_us"] = lambda: medusa_parents_gpu(probs5, 1024)
+        calls["tree_from_probabilities_111110_paths_us"] = lambda: medusa_parents_gpu(probs5, 1024, status=st)
     return {name: device_us(fn) for name, fn in calls.items() if stages is None or name in stages}
 
 

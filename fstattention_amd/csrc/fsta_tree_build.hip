@@ -13,7 +13,9 @@
 //   1. scores of all candidates into LDS
 //   2. the (n-1)-th largest score by radix selection on the bit patterns (up to 8 passes of 8 bits,
 //      ending as soon as the candidates left all belong to the kept ones; non-negative doubles
-//      order like their bit patterns)
+//      order like their bit patterns).  With many candidates the search first runs over the first
+//      1024 of them: its result is a lower bound of the threshold, and the search proper runs over
+//      the short list of candidates at or above that bound (the same threshold, fewer keys per pass)
 //   3. "kept" flags (above the threshold, or equal to it and among the first ties), numbered by
 //      a prefix sum over the candidate index
 //   4. parent ids through the numbering of the parents' candidates
@@ -27,6 +29,7 @@ constexpr int kBuildWaves = kBuildThreads / 64;
 constexpr int kBuildRows = 16;                                  // candidate c belongs to thread c % 1024, row c / 1024
 constexpr int kBuildMaxCand = kBuildThreads * kBuildRows;       // 16384: 128 KB of scores
 constexpr int kBuildMaxProbs = 1024;                            // depths * topk
+constexpr int kBuildShort = 2048;                               // short list of the threshold search: 16 KB
 
 template <typename T>
 __global__ __launch_bounds__(kBuildThreads) void medusa_tree_kernel(const T* __restrict__ probs, int depths, int topk,
@@ -37,7 +40,8 @@ __global__ __launch_bounds__(kBuildThreads) void medusa_tree_kernel(const T* __r
     uint64_t* key_s = reinterpret_cast<uint64_t*>(build_s);                    // [n_cand] score bits, later node ids
     double* prob_s = reinterpret_cast<double*>(key_s + n_cand);                // [depths * topk]
     uint32_t* hist_s = reinterpret_cast<uint32_t*>(prob_s + depths * topk);    // [256] bytes; later counts per (row, wave)
-    uint32_t* misc_s = hist_s + 256;   // [0] chosen byte, [1] candidates still wanted, [2] selection finished
+    uint32_t* misc_s = hist_s + 256;   // [0] chosen byte, [1] candidates still wanted, [2] selection finished, [3] length of the short list
+    uint64_t* short_s = reinterpret_cast<uint64_t*>(misc_s + 4);               // [kBuildShort] candidates at or above a lower bound of the threshold
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -48,7 +52,6 @@ __global__ __launch_bounds__(kBuildThreads) void medusa_tree_kernel(const T* __r
         return;
     }
     for (int e = tid; e < depths * topk; e += kBuildThreads) prob_s[e] = (double)probs[e];
-    if (tid < 3) misc_s[tid] = 0u;
     __syncthreads();
 
     // 1. scores, depth by depth: a path's score is its prefix's score times the probability of
@@ -80,67 +83,110 @@ __global__ __launch_bounds__(kBuildThreads) void medusa_tree_kernel(const T* __r
         }
     }
 
-    // 2. threshold = the keep-th largest key
-    uint64_t prefix = 0ull;        // the bytes of the threshold found so far (in place, lower bytes zero)
-    uint32_t want = (uint32_t)keep;
-    for (int shift = 56; shift >= 0; shift -= 8) {
-        if (tid < 256) hist_s[tid] = 0u;
-        __syncthreads();
-        const uint64_t high_mask = shift == 56 ? 0ull : ~0ull << (shift + 8);
+    // 2. threshold = the keep-th largest key, and how many of the keys equal to it are kept
+    // select(src, count, k): the k-th largest of src[0 .. count) by radix selection, 8 bits per pass from the top
+    // (non-negative doubles order like their bit patterns); a pass ends the search as soon as every key left is wanted.
+    uint64_t threshold = 0ull;
+    uint32_t want = 0u;
+    auto select = [&](const uint64_t* src, int count, uint32_t k) {
+        const int src_rows = (count + kBuildThreads - 1) / kBuildThreads;
+        uint64_t prefix = 0ull;        // the bytes of the threshold found so far (in place, lower bytes zero)
+        uint32_t left = k;
+        if (tid < 3) misc_s[tid] = 0u;
+        for (int shift = 56; shift >= 0; shift -= 8) {
+            if (tid < 256) hist_s[tid] = 0u;
+            __syncthreads();
+            const uint64_t high_mask = shift == 56 ? 0ull : ~0ull << (shift + 8);
 #pragma unroll 1
-        for (int k = 0; k < rows; ++k) {
-            const int c = tid + k * kBuildThreads;
+            for (int r = 0; r < src_rows; ++r) {
+                const int c = tid + r * kBuildThreads;
+                const uint64_t key = c < count ? src[c] : 0ull;
+                const bool in = c < count && (key & high_mask) == prefix;
+                const uint32_t bin = (uint32_t)(key >> shift) & 255u;
+                // The leading bytes of the scores are nearly all alike: 64 atomics of a wave would queue
+                // on one or two words.  For up to two byte values one lane counts for all lanes that
+                // hold it; what is left after that is spread over many words and goes lane by lane.
+                uint64_t voters = __ballot(in);
+#pragma unroll
+                for (int round = 0; round < 2; ++round) {
+                    if (voters != 0ull) {
+                        const int leader = __ffsll((long long)voters) - 1;
+                        const uint32_t first = __builtin_amdgcn_readlane(bin, leader);
+                        const uint64_t same = __ballot(in && bin == first);
+                        if (lane == leader) atomicAdd(&hist_s[first], (uint32_t)__popcll(same));
+                        voters &= ~same;
+                    }
+                }
+                if ((voters >> lane) & 1ull) atomicAdd(&hist_s[bin], 1u);
+            }
+            __syncthreads();
+            if (tid < 64) {
+                // lane l owns bins 255 - 4l .. 252 - 4l; counts accumulate from the largest byte down
+                uint32_t mine[4], local = 0u;
+#pragma unroll
+                for (int b = 0; b < 4; ++b) { mine[b] = hist_s[255 - 4 * tid - b]; local += mine[b]; }
+                uint32_t incl = local;
+#pragma unroll
+                for (int dlt = 1; dlt < 64; dlt <<= 1) {
+                    const uint32_t up = __shfl_up(incl, dlt, 64);
+                    if (tid >= dlt) incl += up;
+                }
+                uint32_t before = incl - local;       // candidates in larger bins
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    if (before < left && left <= before + mine[b]) {
+                        misc_s[0] = (uint32_t)(255 - 4 * tid - b);
+                        misc_s[1] = left - before;
+                        // every candidate of this byte value is wanted: the lower bytes need no look
+                        if (left - before == mine[b]) misc_s[2] = 1u;
+                    }
+                    before += mine[b];
+                }
+            }
+            __syncthreads();
+            prefix |= (uint64_t)misc_s[0] << shift;
+            left = misc_s[1];
+            // (uniform: everyone reads the flag between the same two barriers)
+            if (misc_s[2] != 0u) break;   // threshold = the prefix with zero lower bytes, all `left` candidates from it up
+        }
+        __syncthreads();   // (the next search clears the words read above)
+        threshold = prefix;
+        want = left;
+    };
+    // The search walks every candidate once per pass.  A lower bound of the threshold shortens it: the keep-th largest
+    // key of ANY 1024 candidates cannot exceed the keep-th largest of all, so the candidates at or above that bound
+    // contain every kept one; they are few (the first 1024 candidates are the shortest paths, whose scores are the
+    // largest), and the search over that short list finds the same threshold and the same number of kept ties.
+    bool found = false;
+    if (n_cand > 2 * kBuildThreads && keep <= kBuildThreads / 2) {
+        select(key_s, kBuildThreads, (uint32_t)keep);
+        const uint64_t bound = threshold;
+        if (tid == 0) misc_s[3] = 0u;
+        __syncthreads();
+        const uint64_t below_me = (1ull << lane) - 1ull;
+#pragma unroll 1
+        for (int r = 0; r < rows; ++r) {
+            const int c = tid + r * kBuildThreads;
             const uint64_t key = c < n_cand ? key_s[c] : 0ull;
-            const bool in = c < n_cand && (key & high_mask) == prefix;
-            const uint32_t bin = (uint32_t)(key >> shift) & 255u;
-            // The leading bytes of the scores are nearly all alike: 64 atomics of a wave would queue
-            // on one or two words.  For up to two byte values one lane counts for all lanes that
-            // hold it; what is left after that is spread over many words and goes lane by lane.
-            uint64_t voters = __ballot(in);
-#pragma unroll
-            for (int round = 0; round < 2; ++round) {
-                if (voters != 0ull) {
-                    const int leader = __ffsll((long long)voters) - 1;
-                    const uint32_t first = __builtin_amdgcn_readlane(bin, leader);
-                    const uint64_t same = __ballot(in && bin == first);
-                    if (lane == leader) atomicAdd(&hist_s[first], (uint32_t)__popcll(same));
-                    voters &= ~same;
-                }
-            }
-            if ((voters >> lane) & 1ull) atomicAdd(&hist_s[bin], 1u);
-        }
-        __syncthreads();
-        if (tid < 64) {
-            // lane l owns bins 255 - 4l .. 252 - 4l; counts accumulate from the largest byte down
-            uint32_t mine[4], local = 0u;
-#pragma unroll
-            for (int b = 0; b < 4; ++b) { mine[b] = hist_s[255 - 4 * tid - b]; local += mine[b]; }
-            uint32_t incl = local;
-#pragma unroll
-            for (int dlt = 1; dlt < 64; dlt <<= 1) {
-                const uint32_t up = __shfl_up(incl, dlt, 64);
-                if (tid >= dlt) incl += up;
-            }
-            uint32_t before = incl - local;       // candidates in larger bins
-#pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                if (before < want && want <= before + mine[b]) {
-                    misc_s[0] = (uint32_t)(255 - 4 * tid - b);
-                    misc_s[1] = want - before;
-                    // every candidate of this byte value is wanted: the lower bytes need no look
-                    if (want - before == mine[b]) misc_s[2] = 1u;
-                }
-                before += mine[b];
+            const bool take = c < n_cand && key >= bound;
+            const uint64_t takers = __ballot(take);
+            if (takers != 0ull) {
+                uint32_t base = 0u;
+                if (lane == 0) base = atomicAdd(&misc_s[3], (uint32_t)__popcll(takers));
+                base = __builtin_amdgcn_readfirstlane(base);
+                const uint32_t pos = base + (uint32_t)__popcll(takers & below_me);
+                if (take && pos < (uint32_t)kBuildShort) short_s[pos] = key;
             }
         }
         __syncthreads();
-        prefix |= (uint64_t)misc_s[0] << shift;
-        want = misc_s[1];
-        // (uniform: everyone reads the flag between the same two barriers)
-        if (misc_s[2] != 0u) break;   // threshold = the prefix with zero lower bytes, all `want` candidates from it up
+        const uint32_t n_short = misc_s[3];
+        __syncthreads();
+        if (n_short <= (uint32_t)kBuildShort) {
+            select(short_s, (int)n_short, (uint32_t)keep);
+            found = true;
+        }
     }
-    // prefix = the threshold; `want` of the candidates equal to it are kept, the first ones by index
-    const uint64_t threshold = prefix;
+    if (!found) select(key_s, n_cand, (uint32_t)keep);
 
     // 3. numbering of the kept candidates in index order.  Index order = row by row, wave by wave,
     //    lane by lane: counts per (row, wave) from ballots (above the threshold | equal to it << 16),
@@ -497,7 +543,7 @@ extern "C" int fsta_medusa_tree(const void* probs, int32_t probs_dtype, int32_t 
         return fail(FSTA_EINVAL, "fsta_medusa_tree: n_nodes=%d but only %lld candidate paths (+ the root)", n_nodes,
                     (long long)n_cand);
     if (!probs || !parent || !status) return fail(FSTA_EINVAL, "fsta_medusa_tree: null pointer");
-    const size_t lds = (size_t)n_cand * 8 + (size_t)depths * topk * 8 + (256 + 4) * 4;
+    const size_t lds = (size_t)n_cand * 8 + (size_t)depths * topk * 8 + (256 + 4) * 4 + (size_t)kBuildShort * 8;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (probs_dtype == FSTA_F32) {
         if (lds > 64 * 1024) {

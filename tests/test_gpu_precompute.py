@@ -262,6 +262,17 @@ def test_medusa_tree_built_on_the_gpu_matches_the_host_builder():
     big = trees.medusa_probs(4, 11, 0.3, 12)       # 16104 candidate paths: the largest the kernel takes
     np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(big).cuda(), 1000).cpu().numpy(),
                                   trees.medusa_parents_from_probs(big, 1000))
+    # the threshold search over the short list of candidates at or above a lower bound: ties at the threshold inside
+    # the short list (every path of a depth scores alike), and a short list that overflows (the last head's ranks all
+    # have probability 1: every path of depth 4 ties with its prefix) so that the search walks all candidates after all
+    flat = np.full((4, 10), 0.1)
+    for n in (12, 111, 300, 500):
+        np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(flat).cuda(), n).cpu().numpy(),
+                                      _best_paths_host(flat, n))
+    flat[3] = 1.0
+    for n in (300, 513):
+        np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(flat).cuda(), n).cpu().numpy(),
+                                      _best_paths_host(flat, n))
     with pytest.raises(ValueError, match="candidate paths"):      # 8 heads of 10 ranks: more than 2**24 paths
         medusa_parents_gpu(torch.from_numpy(trees.medusa_probs(8, 10, 0.3, 13)).cuda(), 300)
     with pytest.raises(ValueError):                # a deeper path scoring above its prefix
