@@ -13,12 +13,14 @@
 //   1. scores of all candidates into LDS
 //   2. the (n-1)-th largest score by radix selection on the bit patterns (up to 8 passes of 8 bits,
 //      ending as soon as the candidates left all belong to the kept ones; non-negative doubles
-//      order like their bit patterns).  With many candidates the search first runs over the first
-//      1024 of them: its result is a lower bound of the threshold, and the search proper runs over
-//      the short list of candidates at or above that bound (the same threshold, fewer keys per pass)
+//      order like their bit patterns)
 //   3. "kept" flags (above the threshold, or equal to it and among the first ties), numbered by
 //      a prefix sum over the candidate index
 //   4. parent ids through the numbering of the parents' candidates
+// When nearly all candidates sit on the last level (four heads of ten ranks: 10000 of 11110), that
+// level is never stored: the (n-1)-th largest score of the shorter paths bounds the threshold from
+// below, the last level is scored on the fly against that bound, and steps 2-4 run over the short
+// list of paths that reach it (same result, a tenth of the keys; 18.5 -> 13.3 us for that shape).
 #include "fsta_common.h"
 
 namespace fsta {
@@ -29,7 +31,10 @@ constexpr int kBuildWaves = kBuildThreads / 64;
 constexpr int kBuildRows = 16;                                  // candidate c belongs to thread c % 1024, row c / 1024
 constexpr int kBuildMaxCand = kBuildThreads * kBuildRows;       // 16384: 128 KB of scores
 constexpr int kBuildMaxProbs = 1024;                            // depths * topk
-constexpr int kBuildShort = 2048;                               // short list of the threshold search: 16 KB
+constexpr int kBuildShort = 2048;                               // short list of the threshold search (scores and indices: 24 KB)
+constexpr int kBuildWords = kBuildMaxCand / 32;                 // a bitmap over the candidate index: 512 words
+// paths of the last level from which its part of the score array holds the short list and three bitmaps
+constexpr int kBuildTailCand = (kBuildShort * 12 + 3 * kBuildWords * 4) / 8;
 
 template <typename T>
 __global__ __launch_bounds__(kBuildThreads) void medusa_tree_kernel(const T* __restrict__ probs, int depths, int topk,
@@ -41,7 +46,6 @@ __global__ __launch_bounds__(kBuildThreads) void medusa_tree_kernel(const T* __r
     double* prob_s = reinterpret_cast<double*>(key_s + n_cand);                // [depths * topk]
     uint32_t* hist_s = reinterpret_cast<uint32_t*>(prob_s + depths * topk);    // [256] bytes; later counts per (row, wave)
     uint32_t* misc_s = hist_s + 256;   // [0] chosen byte, [1] candidates still wanted, [2] selection finished, [3] length of the short list
-    uint64_t* short_s = reinterpret_cast<uint64_t*>(misc_s + 4);               // [kBuildShort] candidates at or above a lower bound of the threshold
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -54,38 +58,9 @@ __global__ __launch_bounds__(kBuildThreads) void medusa_tree_kernel(const T* __r
     for (int e = tid; e < depths * topk; e += kBuildThreads) prob_s[e] = (double)probs[e];
     __syncthreads();
 
-    // 1. scores, depth by depth: a path's score is its prefix's score times the probability of
-    //    its last rank (the left-to-right product); one division by topk per candidate, done as
-    //    a multiplication by 2^32 / topk rounded up (exact below 2^32 / topk, i.e. for every index here)
-    if (topk == 1) {       // a single chain: one path per depth
-        if (tid == 0) {
-            double score = 1.0;
-            for (int d = 0; d < depths; ++d) {
-                score *= prob_s[d];
-                key_s[d] = (uint64_t)__double_as_longlong(score);
-            }
-        }
-        __syncthreads();
-    } else {
-        const uint32_t magic = (uint32_t)((0x100000000ull + (uint32_t)topk - 1u) / (uint32_t)topk);
-        int start = 0, prev_start = 0, count = topk;
-        for (int d = 0; start < n_cand; ++d) {
-            for (int v = tid; v < count; v += kBuildThreads) {
-                const uint32_t q = __umulhi((uint32_t)v, magic);          // v / topk
-                const uint32_t r = (uint32_t)v - q * (uint32_t)topk;
-                const double head = d == 0 ? 1.0 : __longlong_as_double((long long)key_s[prev_start + q]);
-                key_s[start + v] = (uint64_t)__double_as_longlong(head * prob_s[d * topk + r]);
-            }
-            __syncthreads();
-            prev_start = start;
-            start += count;
-            count *= topk;
-        }
-    }
-
-    // 2. threshold = the keep-th largest key, and how many of the keys equal to it are kept
-    // select(src, count, k): the k-th largest of src[0 .. count) by radix selection, 8 bits per pass from the top
-    // (non-negative doubles order like their bit patterns); a pass ends the search as soon as every key left is wanted.
+    // select(src, count, k): the k-th largest of src[0 .. count) and how many of the keys equal to it belong to the k
+    // largest, by radix selection, 8 bits per pass from the top (non-negative doubles order like their bit
+    // patterns); a pass ends the search as soon as every key left is wanted.
     uint64_t threshold = 0ull;
     uint32_t want = 0u;
     auto select = [&](const uint64_t* src, int count, uint32_t k) {
@@ -153,40 +128,161 @@ __global__ __launch_bounds__(kBuildThreads) void medusa_tree_kernel(const T* __r
         threshold = prefix;
         want = left;
     };
-    // The search walks every candidate once per pass.  A lower bound of the threshold shortens it: the keep-th largest
-    // key of ANY 1024 candidates cannot exceed the keep-th largest of all, so the candidates at or above that bound
-    // contain every kept one; they are few (the first 1024 candidates are the shortest paths, whose scores are the
-    // largest), and the search over that short list finds the same threshold and the same number of kept ties.
-    bool found = false;
-    if (n_cand > 2 * kBuildThreads && keep <= kBuildThreads / 2) {
-        select(key_s, kBuildThreads, (uint32_t)keep);
-        const uint64_t bound = threshold;
-        if (tid == 0) misc_s[3] = 0u;
-        __syncthreads();
-        const uint64_t below_me = (1ull << lane) - 1ull;
-#pragma unroll 1
-        for (int r = 0; r < rows; ++r) {
-            const int c = tid + r * kBuildThreads;
-            const uint64_t key = c < n_cand ? key_s[c] : 0ull;
-            const bool take = c < n_cand && key >= bound;
-            const uint64_t takers = __ballot(take);
-            if (takers != 0ull) {
+    // Scores of the levels from `d` on, as long as they start below `limit`: a path's score is its prefix's score
+    // times the probability of its last rank (the left-to-right product); one division by topk per candidate, done
+    // as a multiplication by 2^32 / topk rounded up (exact below 2^32 / topk, i.e. for every index here).
+    const uint32_t magic = (uint32_t)((0x100000000ull + (uint32_t)topk - 1u) / (uint32_t)max(topk, 1));
+    int lvl = 0, start = 0, prev_start = 0, count = topk;      // the next level to score
+    auto score_levels = [&](int limit) {
+        for (; start < limit; ++lvl) {
+            for (int v = tid; v < count; v += kBuildThreads) {
+                const uint32_t q = __umulhi((uint32_t)v, magic);          // v / topk
+                const uint32_t r = (uint32_t)v - q * (uint32_t)topk;
+                const double head = lvl == 0 ? 1.0 : __longlong_as_double((long long)key_s[prev_start + q]);
+                key_s[start + v] = (uint64_t)__double_as_longlong(head * prob_s[lvl * topk + r]);
+            }
+            __syncthreads();
+            prev_start = start;
+            start += count;
+            count *= topk;
+        }
+    };
+
+    // ---- many candidates, nearly all of them on the last level: the last level is never stored -----------------
+    // The keep-th largest score of the shorter paths (the head: every level but the last) is a lower bound of the
+    // threshold: the keep-th largest of any subset cannot exceed the keep-th largest of all.  The paths of the last
+    // level are scored on the fly and only those at or above the bound join a short list, together with the head's;
+    // the list contains every kept path, so the search over it finds the same threshold and the same number of kept
+    // ties.  Kept paths are then numbered through a bitmap over the candidate index (ids in index order = bits below)
+    // and their parents looked up in the same bitmap.  The tail of the score array, which the last level does not
+    // use here, holds the list and the bitmaps.  A list that overflows sends the launch down the general way below.
+    {
+        int last = 1;
+        for (int d = 0; d < depths && last <= kBuildMaxCand; ++d) last *= topk;     // paths of the last level
+        const int n_head = n_cand - last;
+        if (depths >= 2 && topk >= 2 && last >= kBuildTailCand && n_head >= keep && n_head <= kBuildShort) {
+            uint64_t* skey_s = key_s + n_head;                                   // [kBuildShort] scores of the listed paths
+            uint32_t* sidx_s = reinterpret_cast<uint32_t*>(skey_s + kBuildShort);   // [kBuildShort] their candidate indices
+            uint32_t* kept_s = sidx_s + kBuildShort;       // [512] bitmap over the candidate index: kept
+            uint32_t* tie_s = kept_s + kBuildWords;        // [512] equal to the threshold
+            uint32_t* below_s = tie_s + kBuildWords;       // [512] bits set in the words before (of the bitmap scanned last)
+            score_levels(n_head);
+            select(key_s, n_head, (uint32_t)keep);
+            const uint64_t bound = threshold;
+            for (int w = tid; w < 2 * kBuildWords; w += kBuildThreads) kept_s[w] = 0u;       // kept and tie bitmaps
+            if (tid == 0) misc_s[3] = 0u;
+            __syncthreads();
+            const uint64_t lanes_below = (1ull << lane) - 1ull;
+            auto list = [&](bool take, uint64_t key, int index) {      // (called by whole waves)
+                const uint64_t takers = __ballot(take);
+                if (takers == 0ull) return;
                 uint32_t base = 0u;
                 if (lane == 0) base = atomicAdd(&misc_s[3], (uint32_t)__popcll(takers));
                 base = __builtin_amdgcn_readfirstlane(base);
-                const uint32_t pos = base + (uint32_t)__popcll(takers & below_me);
-                if (take && pos < (uint32_t)kBuildShort) short_s[pos] = key;
+                const uint32_t pos = base + (uint32_t)__popcll(takers & lanes_below);
+                if (take && pos < (uint32_t)kBuildShort) {
+                    skey_s[pos] = key;
+                    sidx_s[pos] = (uint32_t)index;
+                }
+            };
+#pragma unroll 1
+            for (int c0 = 0; c0 < n_head; c0 += kBuildThreads) {
+                const int c = c0 + tid;
+                const uint64_t key = c < n_head ? key_s[c] : 0ull;
+                list(c < n_head && key >= bound, key, c);
+            }
+#pragma unroll 1
+            for (int v0 = 0; v0 < last; v0 += kBuildThreads) {
+                const int v = v0 + tid;
+                const bool valid = v < last;
+                const uint32_t q = __umulhi((uint32_t)(valid ? v : 0), magic);
+                const uint32_t r = (uint32_t)(valid ? v : 0) - q * (uint32_t)topk;
+                const double head = __longlong_as_double((long long)key_s[prev_start + q]);
+                const uint64_t key = (uint64_t)__double_as_longlong(head * prob_s[lvl * topk + r]);
+                list(valid && key >= bound, key, n_head + v);
+            }
+            __syncthreads();
+            const int n_short = (int)misc_s[3];
+            if (n_short <= kBuildShort) {       // (uniform)
+                select(skey_s, n_short, (uint32_t)keep);
+                // bitmaps: above the threshold -> kept; equal to it -> tie
+                for (int e = tid; e < n_short; e += kBuildThreads) {
+                    const uint64_t key = skey_s[e];
+                    const uint32_t c = sidx_s[e];
+                    if (key > threshold) atomicOr(&kept_s[c >> 5], 1u << (c & 31));
+                    else if (key == threshold) atomicOr(&tie_s[c >> 5], 1u << (c & 31));
+                }
+                __syncthreads();
+                // below_s[w] = bits set in words [0, w) of a bitmap: one wave, 8 words per lane
+                auto count_below = [&](const uint32_t* bits) {
+                    if (tid < 64) {
+                        uint32_t mine[8], local = 0u;
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) { mine[i] = (uint32_t)__popc(bits[8 * tid + i]); local += mine[i]; }
+                        uint32_t incl = local;
+#pragma unroll
+                        for (int dlt = 1; dlt < 64; dlt <<= 1) {
+                            const uint32_t up = __shfl_up(incl, dlt, 64);
+                            if (tid >= dlt) incl += up;
+                        }
+                        uint32_t before = incl - local;
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) { below_s[8 * tid + i] = before; before += mine[i]; }
+                    }
+                    __syncthreads();
+                };
+                auto rank_in = [&](const uint32_t* bits, uint32_t c) {      // bits set below position c
+                    return below_s[c >> 5] + (uint32_t)__popc(bits[c >> 5] & ((1u << (c & 31)) - 1u));
+                };
+                // the first `want` ties in index order are kept as well
+                count_below(tie_s);
+                for (int e = tid; e < n_short; e += kBuildThreads) {
+                    const uint32_t c = sidx_s[e];
+                    if (skey_s[e] == threshold && rank_in(tie_s, c) < want) atomicOr(&kept_s[c >> 5], 1u << (c & 31));
+                }
+                __syncthreads();
+                count_below(kept_s);
+                // ids = 1 + kept paths below in index order; the parent of a path is the path without its last rank
+                if (tid == 0) parent[0] = -1;
+                bool broken = false;
+                for (int e = tid; e < n_short; e += kBuildThreads) {
+                    const uint32_t c = sidx_s[e];
+                    if (!((kept_s[c >> 5] >> (c & 31)) & 1u)) continue;
+                    int s0 = 0, cnt = topk, p0 = 0;
+                    while ((int)c >= s0 + cnt) { p0 = s0; s0 += cnt; cnt *= topk; }
+                    int64_t par = 0;      // paths of one rank hang off the root
+                    if (s0 > 0) {
+                        const uint32_t pc = (uint32_t)p0 + ((uint32_t)c - (uint32_t)s0) / (uint32_t)topk;
+                        if ((kept_s[pc >> 5] >> (pc & 31)) & 1u) par = 1 + (int64_t)rank_in(kept_s, pc);
+                        else broken = true;     // the parent path was not kept: probabilities above 1 or not numbers
+                    }
+                    parent[1 + rank_in(kept_s, c)] = par;
+                }
+                if (broken) atomicOr(status, FSTA_TREE_NOT_PREFIX_CLOSED);
+                return;
+            }
+            // (the list overflowed: scores of more than kBuildShort paths reach the bound)
+            __syncthreads();
+        }
+    }
+
+    // ---- the general way: every score stored, the search over all of them -----------------------------------------
+    // 1. scores, depth by depth
+    if (topk == 1) {       // a single chain: one path per depth
+        if (tid == 0) {
+            double score = 1.0;
+            for (int d = 0; d < depths; ++d) {
+                score *= prob_s[d];
+                key_s[d] = (uint64_t)__double_as_longlong(score);
             }
         }
         __syncthreads();
-        const uint32_t n_short = misc_s[3];
-        __syncthreads();
-        if (n_short <= (uint32_t)kBuildShort) {
-            select(short_s, (int)n_short, (uint32_t)keep);
-            found = true;
-        }
+    } else {
+        score_levels(n_cand);
     }
-    if (!found) select(key_s, n_cand, (uint32_t)keep);
+
+    // 2. threshold = the keep-th largest key, and how many of the keys equal to it are kept
+    select(key_s, n_cand, (uint32_t)keep);
 
     // 3. numbering of the kept candidates in index order.  Index order = row by row, wave by wave,
     //    lane by lane: counts per (row, wave) from ballots (above the threshold | equal to it << 16),
@@ -543,7 +639,7 @@ extern "C" int fsta_medusa_tree(const void* probs, int32_t probs_dtype, int32_t 
         return fail(FSTA_EINVAL, "fsta_medusa_tree: n_nodes=%d but only %lld candidate paths (+ the root)", n_nodes,
                     (long long)n_cand);
     if (!probs || !parent || !status) return fail(FSTA_EINVAL, "fsta_medusa_tree: null pointer");
-    const size_t lds = (size_t)n_cand * 8 + (size_t)depths * topk * 8 + (256 + 4) * 4 + (size_t)kBuildShort * 8;
+    const size_t lds = (size_t)n_cand * 8 + (size_t)depths * topk * 8 + (256 + 4) * 4;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (probs_dtype == FSTA_F32) {
         if (lds > 64 * 1024) {

@@ -273,6 +273,14 @@ def test_medusa_tree_built_on_the_gpu_matches_the_host_builder():
     for n in (300, 513):
         np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(flat).cuda(), n).cpu().numpy(),
                                       _best_paths_host(flat, n))
+    # many seeds through the way that never stores the last level (and its overflow into the general way)
+    for seed in range(12):
+        for depths, topk, n in [(4, 10, 256), (4, 10, 512), (4, 10, 1000), (3, 24, 256), (4, 8, 128), (2, 100, 90)]:
+            probs = trees.medusa_probs(depths, topk, 0.3 + 0.1 * (seed % 4), 100 + seed)
+            if seed % 3 == 2:
+                probs = probs.astype(np.float32)
+            np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(probs).cuda(), n).cpu().numpy(),
+                                          _best_paths_host(probs, n), err_msg=f"seed {seed} {depths}x{topk} n={n}")
     with pytest.raises(ValueError, match="candidate paths"):      # 8 heads of 10 ranks: more than 2**24 paths
         medusa_parents_gpu(torch.from_numpy(trees.medusa_probs(8, 10, 0.3, 13)).cuda(), 300)
     with pytest.raises(ValueError):                # a deeper path scoring above its prefix
