@@ -366,6 +366,23 @@ def test_non_positive_scale(scale):
         run_tree(parent, 64, 1, 2, 64, dtype, 13, scale=scale)
 
 
+@pytest.mark.parametrize("n,block_m,heads,dtype", [(700, 64, 30, torch.bfloat16), (900, 128, 40, torch.float16),
+                                                   (1000, 64, 32, torch.bfloat16)])
+def test_launches_of_one_to_two_workgroups_per_cu(n, block_m, heads, dtype):
+    # more than 256 and at most 512 workgroups: the late blocks of every slice are dispatched first; a ragged last
+    # block, a head count that does not fill the last group of eight slices, every row against the dense oracle
+    parent = trees.random_recursive_parents(n, 17, window=48)
+    a_idx, a_mask, l_idx, max_anc = oracle_inputs(parent, block_m)
+    q, k, v = rand_qkv(1, heads, n, n, 128, dtype, 23)
+    scale = 1.0 / math.sqrt(128)
+    want, _ = dense_oracle(q, k, v, parent, scale)
+    o = fst_attention(q.cuda(), k.cuda(), v.cuda(), a_idx.cuda(), a_mask.cuda(), l_idx.cuda(), scale,
+                      BLOCK_M=block_m, MAX_ANCESTORS=max_anc, out_dtype=torch.float32)
+    from fstattention_amd import _lib
+    assert "attn_mfma16_kernel" in _lib.load().fsta_last_attention_kernel().decode()
+    assert_close(o, want, dtype, f"n={n} m={block_m} heads={heads}")
+
+
 def test_ragged_query_count():
     # nq not a multiple of block_m: rows past nq are neither read nor written
     parent = trees.random_recursive_parents(100, 3)
