@@ -281,6 +281,13 @@ def test_medusa_tree_built_on_the_gpu_matches_the_host_builder():
                 probs = probs.astype(np.float32)
             np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(probs).cuda(), n).cpu().numpy(),
                                           _best_paths_host(probs, n), err_msg=f"seed {seed} {depths}x{topk} n={n}")
+    # a last-level rank with a "probability" above 1: paths of depth 4 outrank their own prefixes, some kept paths have
+    # no kept parent (they hang off the root, as in the host's table of ids) and the status word says so
+    odd = trees.medusa_probs(4, 10, 0.3, 77)
+    odd[3, 0] = 40.0
+    np.testing.assert_array_equal(medusa_parents_gpu(torch.from_numpy(odd).cuda(), 256).cpu().numpy(), _best_paths_host(odd, 256))
+    with pytest.raises(ValueError):
+        medusa_parents_gpu(torch.from_numpy(odd).cuda(), 256, check=True)
     with pytest.raises(ValueError, match="candidate paths"):      # 8 heads of 10 ranks: more than 2**24 paths
         medusa_parents_gpu(torch.from_numpy(trees.medusa_probs(8, 10, 0.3, 13)).cuda(), 300)
     with pytest.raises(ValueError):                # a deeper path scoring above its prefix
