@@ -339,6 +339,16 @@ def test_short_ancestor_lists_both_wave_pairings(block_m, d, dtype, share_tiles)
     run_tree(bushy, block_m, 2, 2, d, dtype, 18, share_tiles=share_tiles)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("scale", [1.5, 6.0])
+def test_two_tiles_per_step_with_peaked_weights(dtype, scale):
+    """The waves that share the head dimension take two ancestor tiles in one step; scores far apart (a large
+    softmax scale) send them through the full update of the running maximum over both tiles."""
+    parent = trees.medusa_parents(n=256, seed=901)
+    run_tree(parent, 64, 1, 6, 128, dtype, 31, scale=scale, want_kernel="-2")
+    run_tree(parent, 128, 1, 3, 64, dtype, 32, scale=scale, want_kernel="-2")
+
+
 def test_reference_test_shape_with_and_without_prefix():
     # the reference's own test: Z=2 H=2 N_CTX=2048 D=64 fp16, tree of 2044 nodes,
     # blocks of 128, 64 ancestors, sm_scale 0.5, inputs N(0, 0.5^2), prefix 0 or 2048
