@@ -240,7 +240,8 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         }
     }
     // Q rows of this wave: whole rows straight into LDS, K-tile swizzle, parked in the last ring
-    // slots until the fragments have been read (before the first barrier).  Rows past the end of
+    // slots until the fragments have been read; the first tiles are requested into the other slots
+    // as soon as the plan is there, without waiting for the Q rows.  Rows past the end of
     // a ragged last block are read as the last row and never stored.
     const int q_row = lane / kCpr, q_slot = lane % kCpr;           // Q rows are 16-bit
     const int dma_row = lane / kKvCpr, dma_slot = lane % kKvCpr;   // K/V rows as stored
@@ -355,8 +356,10 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         if (gathers && n_spec) wait_vmcnt<kQDma + kEarlyTiles * kDmaPerWave>();
         else wait_vmcnt<kQDma>();
     } else {
-        read_q(0);        // Q sits in ring slots the gathers are about to take (waits for all of this wave's transfers)
-        ring_barrier();   // everybody's pieces of the plan have landed, everybody has read its Q rows
+        // the plan has landed (it usually comes from L2: every slice reads the same one); the Q rows, which come
+        // from HBM, stay in flight while the first tiles are requested into the ring slots Q does not occupy
+        wait_vmcnt<kQDma>();
+        ring_barrier();   // everybody's pieces of the plan have landed
     }
     FSTA_STAMP(2);    // the plan is here
     // From the plan: ancestor count, validity of this lane's own leaf slot and, after early leaf
@@ -538,6 +541,13 @@ __global__ __launch_bounds__(M * 4 * (KS < 0 ? -KS : KS), 4) void attn_mfma16_ke
         __syncthreads();
         issued = consumed;
         issue_slot = 0;
+    }
+    if (!early_leaf) {
+        // (Q is parked in the last ring slots -- 8-bit K/V: in the widened tiles, the whole staging ring is free)
+        constexpr int kQSlots = KV8 ? 0 : (kWaves * 16 + 2 * kTileN - 1) / (2 * kTileN);
+        refill_to(consumed + stages - kQSlots);
+        read_q(issued - consumed);
+        ring_barrier();   // everybody has read its Q rows: their slots are free
     }
     refill();
     FSTA_STAMP(3);    // ancestor tiles requested
